@@ -47,5 +47,9 @@ from .gegorax import GegoraxRingModel  # noqa: E402
 
 register(GegoraxRingModel)
 
-__all__ = ["GegoraxRingModel", "ModelConfig", "QuantConfig", "RingModel", "MoERingModel", "KVCache", "PosudraRingModel",
+from .komizen import KomizenRingModel  # noqa: E402
+
+register(KomizenRingModel)
+
+__all__ = ["GegoraxRingModel", "KomizenRingModel", "ModelConfig", "QuantConfig", "RingModel", "MoERingModel", "KVCache", "PosudraRingModel",
            "Linear", "PRESETS", "get_ring_model", "register"]

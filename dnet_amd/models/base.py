@@ -311,11 +311,13 @@ class KVCache:
             # layer -> per-layer tensors [B, Hkv_l, Smax, D_l] (self.k[li]
             # indexes a list instead of a stacked tensor's first axis); a
             # layer without attention has None
+            # v_dim 0: the layer's values are a leading slice of its key
+            # rows (latent attention) and only k[li] exists
             assert kv_bits == 16 and len(layer_dims) == L
             self.k = [None if t is None else
                       torch.zeros(batch, t[0], smax, t[1], dtype=dtype,
                                   device=device) for t in layer_dims]
-            self.v = [None if t is None else
+            self.v = [None if t is None or not t[2] else
                       torch.zeros(batch, t[0], smax, t[2], dtype=dtype,
                                   device=device) for t in layer_dims]
             return
@@ -527,6 +529,12 @@ class RingModel:
     # (executor buffers and ring hops follow it) and of its logits
     act_dtype = torch.bfloat16
     logits_dtype = torch.bfloat16
+
+    @property
+    def hidden_width(self) -> int:
+        """Row width of the residual between windows and pipeline stages."""
+        return self.cfg.hidden_size
+
     supports_float32 = False      # cfg.compute_dtype == "float32" honoured
     # prefill_window accepts per-row start positions / lengths (ragged
     # batches of unequal prompts in one call)

@@ -72,6 +72,13 @@ class ModelConfig:
     # per-layer token input (gegorax): width of each layer's slice of the
     # second embedding table; 0 = none
     token_side_dim: int = 0
+    # layer loops (komizen): layer run i uses the stored weights of layer
+    # layer_weight_ids[i] (a looped span repeats its ids; every run has its
+    # own cache / state); None = run i uses layer i
+    layer_weight_ids: Optional[list] = None
+    # hyper-connections (komizen): number of residual streams a layer mixes
+    # (0 = one plain residual)
+    hc_streams: int = 0
     # "bfloat16": bf16 weights/activations with 32-bit accumulation;
     # "float32": weights, activations and matrix products in true fp32
     # (honoured by the model families that implement it)
@@ -80,6 +87,13 @@ class ModelConfig:
     @property
     def qkv_out(self) -> int:
         return (self.num_q_heads + 2 * self.num_kv_heads) * self.head_dim
+
+    def stored_layers(self, layer_ids) -> list:
+        """Ids of the checkpoint layers whose tensors the given layer runs
+        read (sorted, each once)."""
+        if self.layer_weight_ids is None:
+            return list(layer_ids)
+        return sorted({self.layer_weight_ids[l] for l in layer_ids})
 
     @classmethod
     def from_posudra(cls, cfg: dict,
@@ -183,12 +197,94 @@ class ModelConfig:
         )
 
     @classmethod
+    def from_komizen(cls, cfg: dict,
+                     quant: Optional[QuantConfig] = None) -> "ModelConfig":
+        """Komizen checkpoints list their layers: {"architecture":
+        "Komizen", "vocab", "width", "norm": {"eps"}, "embedding":
+        {"scale"}, "streams" (optional), "loop": {"start", "stop", "times"}
+        (optional), "layers": [{"type": "delta" | "mamba2" |
+        "latent_attention", "mixer": {...}, "mlp": {"kind": "moe", ...} |
+        null}, ...]}. A looped span of layers is unrolled here: the model
+        then holds one layer run per pass (``num_layers`` counts runs) and
+        ``layer_weight_ids`` names the stored layer each run reads."""
+        need = {"delta": ("conv", "dim", "heads", "kv_heads", "vdim"),
+                "mamba2": ("conv", "groups", "heads", "norm_groups", "state",
+                           "vdim"),
+                "latent_attention": ("dim", "heads", "kv_rank", "q_rank",
+                                     "rot", "rot_dim", "scale", "vdim")}
+        stored = [dict(s) for s in cfg["layers"]]
+        for i, s in enumerate(stored):
+            kind, m = s.get("type"), s.get("mixer") or {}
+            if kind not in need:
+                raise ValueError(f"komizen layer {i}: unknown mixer type "
+                                 f"{kind!r}")
+            missing = [k for k in need[kind] if k not in m]
+            if missing:
+                raise ValueError(f"komizen layer {i}: mixer lacks {missing}")
+            if kind == "delta" and m["heads"] % m["kv_heads"]:
+                raise ValueError(f"komizen layer {i}: heads % kv_heads")
+            if kind == "mamba2" and (
+                    m["heads"] % m["groups"]
+                    or (m["heads"] * m["vdim"]) % m["norm_groups"]):
+                raise ValueError(f"komizen layer {i}: head counts do not "
+                                 "divide")
+            if kind == "latent_attention":
+                rot = m["rot"]
+                if int(rot["dims"]) != int(m["rot_dim"]) \
+                        or int(rot["dims"]) % 2:
+                    raise ValueError(f"komizen layer {i}: rot.dims must be "
+                                     "the (even) rotated size")
+            ff = s.get("mlp")
+            if ff is not None:
+                if ff.get("kind") != "moe":
+                    raise ValueError(f"komizen layer {i}: unknown "
+                                     f"feed-forward kind {ff.get('kind')!r}")
+                if not 0 < ff["router"]["top"] <= ff["router"]["experts"]:
+                    raise ValueError(f"komizen layer {i}: router.top")
+        ids = list(range(len(stored)))
+        loop = cfg.get("loop")
+        if loop:
+            a, b, k = int(loop["start"]), int(loop["stop"]), \
+                int(loop["times"])
+            if not (0 <= a <= b <= len(stored)) or k < 1:
+                raise ValueError("komizen: loop span out of range")
+            ids = ids[:a] + ids[a:b] * k + ids[b:]
+        specs = [stored[i] for i in ids]
+        att = next((s["mixer"] for s in specs
+                    if s["type"] == "latent_attention"), {})
+        moe = [s["mlp"] for s in specs if s.get("mlp")]
+        return cls(
+            model_type="komizen",
+            hidden_size=cfg["width"],
+            num_layers=len(specs),
+            num_q_heads=att.get("heads", 1),
+            num_kv_heads=1,
+            head_dim=att.get("dim", 1),
+            v_head_dim=att.get("vdim", 1),
+            intermediate_size=0,
+            num_experts=max((m["router"]["experts"] for m in moe), default=0),
+            num_experts_per_tok=max((m["router"]["top"] for m in moe),
+                                    default=0),
+            vocab_size=cfg["vocab"],
+            rms_eps=cfg["norm"]["eps"],
+            embedding_scale=float((cfg.get("embedding") or {}).get("scale",
+                                                                   1.0)),
+            tie_word_embeddings=True,
+            layer_specs=specs,
+            layer_weight_ids=ids,
+            hc_streams=int(cfg.get("streams") or 0),
+            quant=quant,
+        )
+
+    @classmethod
     def from_hf(cls, cfg: dict, quant: Optional[QuantConfig] = None) -> "ModelConfig":
         arch = str(cfg.get("architecture", "")).lower()
         if arch == "posudra" or cfg.get("model_type") == "posudra":
             return cls.from_posudra(cfg, quant)
         if arch == "gegorax" or cfg.get("model_type") == "gegorax":
             return cls.from_gegorax(cfg, quant)
+        if arch == "komizen" or cfg.get("model_type") == "komizen":
+            return cls.from_komizen(cfg, quant)
         mt = cfg.get("model_type", "llama")
         hidden = cfg["hidden_size"]
         nq = cfg.get("num_attention_heads", 32)
@@ -297,6 +393,52 @@ def gegorax_config(width: int, layers: int, vocab: int, heads: int,
     return cfg
 
 
+def komizen_config(width: int, vocab: int, pattern: str = "ldm",
+                   layers: int = 0, heads: int = 4, dim: int = 32,
+                   rot_dim: int = 16, vdim: int = 32, kv_rank: int = 64,
+                   q_rank: int = 48, delta_heads: int = 4,
+                   delta_kv_heads: int = 2, delta_dim: int = 16,
+                   delta_vdim: int = 32, ssm_heads: int = 4,
+                   ssm_vdim: int = 16, ssm_state: int = 16,
+                   ssm_groups: int = 1, norm_groups: int = 1, conv: int = 4,
+                   experts: int = 4, top: int = 2, expert_ff: int = 64,
+                   router_scale: float = 1.0, streams: int = 2,
+                   loop: Optional[tuple] = None, rot_base: float = 10000.0,
+                   eps: float = 1e-6, embedding_scale: float = 1.0) -> dict:
+    """A komizen stack in the checkpoint's config.json layout. ``pattern``
+    repeats over the ``layers`` stored layers (default: once): 'l' = latent
+    attention, 'd' = gated delta rule, 'm' = mamba2; every layer has a
+    mixture-of-experts feed-forward when ``experts`` > 0. ``loop`` =
+    (start, stop, times)."""
+    mix = {
+        "l": ("latent_attention",
+              {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim,
+               "kv_rank": kv_rank, "q_rank": q_rank,
+               "scale": (dim + rot_dim) ** -0.5,
+               "rot": {"base": rot_base, "dims": rot_dim}}),
+        "d": ("delta", {"heads": delta_heads, "kv_heads": delta_kv_heads,
+                        "dim": delta_dim, "vdim": delta_vdim, "conv": conv}),
+        "m": ("mamba2", {"heads": ssm_heads, "vdim": ssm_vdim,
+                         "state": ssm_state, "groups": ssm_groups,
+                         "norm_groups": norm_groups, "conv": conv}),
+    }
+    ff = ({"kind": "moe", "expert": {"ff": expert_ff},
+           "router": {"experts": experts, "top": top, "scale": router_scale}}
+          if experts else None)
+    out = []
+    for i in range(layers or len(pattern)):
+        kind, m = mix[pattern[i % len(pattern)]]
+        out.append({"type": kind, "mixer": dict(m), "mlp": ff})
+    cfg = {"architecture": "Komizen", "vocab": vocab, "width": width,
+           "norm": {"eps": eps}, "embedding": {"scale": embedding_scale},
+           "layers": out}
+    if streams:
+        cfg["streams"] = streams
+    if loop:
+        cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return cfg
+
+
 # Known configs for synthetic benchmarking (random-init weights; no network).
 PRESETS: dict[str, dict] = {
     "llama-3-8b": dict(model_type="llama", hidden_size=4096, num_hidden_layers=32,
@@ -362,6 +504,8 @@ PRESETS: dict[str, dict] = {
     "gegorax-tiny": gegorax_config(128, 4, 256, 4, 2, 32, 16, 24, 4, 4, 16,
                                    16, 2, 32, 192, experts=6, top=2,
                                    expert_ff=64, shared_ff=64, side_dim=16),
+    "komizen-tiny": komizen_config(128, 256, "ldm", layers=4, loop=(1, 3, 2),
+                                   embedding_scale=4.0),
     "tiny": dict(model_type="llama", hidden_size=128, num_hidden_layers=4,
                  num_attention_heads=2, num_key_value_heads=2, head_dim=64,
                  intermediate_size=256, vocab_size=256, rope_theta=10000.0),

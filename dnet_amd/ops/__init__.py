@@ -512,19 +512,23 @@ def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
              pos: torch.Tensor, T: int, scale: float, lens=None, slots=None,
              temp=None, softcap: float = 0.0, dist_r1=None, dist_r2=None,
              sinks=None, window: int = 0, pool_k=None, pool_v=None,
-             pool: int = 0) -> torch.Tensor:
+             pool: int = 0, v_dim: int = 0) -> torch.Tensor:
     """Causal attention against the cache with per-head temperature, tanh
     soft cap, logarithmic distance penalty and a sink in the softmax
     denominator (each optional). One entry point for decode (T=1) and
     ragged batched prefill (T = padded length, lens = real lengths).
     ``window`` > 0 limits the tokens seen to the last ``window``; with
     ``pool`` > 0 every whole block of ``pool`` positions before the window
-    is seen as one entry of the pooled caches (see ``kv_pool_update``)."""
+    is seen as one entry of the pooled caches (see ``kv_pool_update``).
+    ``vcache`` None (latent attention): the values are the first ``v_dim``
+    entries of the key rows, which the kernels then stage once for both."""
     if pool:
         assert window and pool_k is not None and pool_v is not None
+    if vcache is None:
+        assert 0 < v_dim <= kcache.shape[3] and not pool
     if q.is_cuda:
         Hkv, D = kcache.shape[1], kcache.shape[3]
-        Dv = vcache.shape[3]
+        Dv = vcache.shape[3] if vcache is not None else v_dim
         Hq = q.shape[1] // D
         # padded rows of a ragged batch are never written by the kernel
         out = (torch.zeros if lens is not None else torch.empty)(
@@ -545,11 +549,11 @@ def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
                            scale, temp, softcap or 0.0, dist_r1, dist_r2,
                            sinks, window or 0, partials, splits,
                            pool_k if pool else None,
-                           pool_v if pool else None, pool or 0)
+                           pool_v if pool else None, pool or 0, Dv)
         return out
     return ref.attn_mod(q, kcache, vcache, pos, T, scale, lens, slots, temp,
                         softcap, dist_r1, dist_r2, sinks, window, pool_k,
-                        pool_v, pool)
+                        pool_v, pool, v_dim)
 
 
 # ---- pooled-block caches, short convolutions, linear recurrences ----
@@ -661,3 +665,81 @@ def clamped_glu(gu: torch.Tensor, alpha: float, limit: float) -> torch.Tensor:
         _native().clamped_glu(gu, y, alpha, limit)
         return y
     return ref.clamped_glu(gu, alpha, limit)
+
+
+# ---- residual streams, gated delta rule, latent attention (komizen) ----
+# csrc/streams.hip.cpp, csrc/gated_delta.hip.cpp, csrc/latent.hip.cpp. The
+# streams, the recurrent state, unit norms, decays and angles are fp32
+# whatever the activation dtype.
+
+def hc_read_norm(xs, w_in, wn, eps: float,
+                 out_dtype: torch.dtype) -> torch.Tensor:
+    if xs.is_cuda:
+        S = w_in.numel()
+        y = torch.empty(xs.shape[0], xs.shape[1] // S, dtype=out_dtype,
+                        device=xs.device)
+        _native().hc_write_read(xs, None, None, None, w_in, wn, y, eps)
+        return y
+    return ref.hc_read_norm(xs, w_in, wn, eps, out_dtype)
+
+
+def hc_write(xs, y, mix, w_out, next_in, next_wn, eps: float,
+             out_dtype: torch.dtype):
+    """Streams xs fp32 [M, S*W] (in place): x_t <- sum_s mix[s,t] x_s +
+    w_out[t] y; returns the next sublayer's normalized read when
+    ``next_in`` / ``next_wn`` are given — one kernel per sublayer boundary."""
+    if xs.is_cuda:
+        assert xs.dtype == torch.float32 and xs.is_contiguous()
+        S = w_out.numel()
+        nxt = (torch.empty(xs.shape[0], xs.shape[1] // S, dtype=out_dtype,
+                           device=xs.device) if next_in is not None else None)
+        _native().hc_write_read(xs, y, mix, w_out, next_in, next_wn, nxt, eps)
+        return nxt
+    return ref.hc_write(xs, y, mix, w_out, next_in, next_wn, eps, out_dtype)
+
+
+def gated_delta_scan(qkv, gates, b_col0: int, a_col0: int, a_log, dt_bias,
+                     state, pos, T: int, H: int, KH: int, d: int, dv: int,
+                     unit_eps: float, lens=None, slots=None) -> torch.Tensor:
+    if qkv.is_cuda:
+        o = (torch.zeros if lens is not None else torch.empty)(
+            qkv.shape[0], H * dv, dtype=torch.float32, device=qkv.device)
+        _native().gated_delta_scan(qkv, gates, b_col0, a_col0, a_log, dt_bias,
+                                   state, o, pos, lens, slots, T, H, KH, d,
+                                   dv, unit_eps)
+        return o
+    return ref.gated_delta_scan(qkv, gates, b_col0, a_col0, a_log, dt_bias,
+                                state, pos, T, H, KH, d, dv, unit_eps, lens,
+                                slots)
+
+
+def latent_append(src, col0: int, wn, eps: float, R: int, rot_freq, kcache,
+                  pos, T: int, lens=None, slots=None) -> None:
+    if src.is_cuda:
+        _native().latent_append(src, col0, wn, eps, R, rot_freq, kcache, pos,
+                                lens, slots, T)
+        return
+    ref.latent_append(src, col0, wn, eps, R, rot_freq, kcache, pos, T, lens,
+                      slots)
+
+
+def latent_q_pack(q, qabs, rot_freq, pos, T: int, H: int,
+                  d: int) -> torch.Tensor:
+    if q.is_cuda:
+        rd = 2 * rot_freq.numel()
+        out = torch.empty(q.shape[0], H * (qabs.shape[2] + rd),
+                          dtype=q.dtype, device=q.device)
+        _native().latent_q_pack(q, qabs, rot_freq, pos, out, T, H, d)
+        return out
+    return ref.latent_q_pack(q, qabs, rot_freq, pos, T, H, d)
+
+
+def moe_up_act(x, w, we) -> torch.Tensor:
+    """Ungated experts, first half: act [E, M, I] = relu(x w_e^T)^2 (bf16;
+    experts with all-zero ``we`` are skipped on the GPU)."""
+    if x.is_cuda:
+        act = torch.empty(w.shape[0], x.shape[0], w.shape[1],
+                          dtype=torch.bfloat16, device=x.device)
+        _native().moe_up_act(x, w, we, act)
+        return act
+    return ref.moe_up_act(x, w, we)

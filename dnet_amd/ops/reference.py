@@ -586,7 +586,7 @@ def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
              pos: torch.Tensor, T: int, scale: float, lens=None, slots=None,
              temp=None, softcap: float = 0.0, dist_r1=None, dist_r2=None,
              sinks=None, window: int = 0, pool_k=None, pool_v=None,
-             pool: int = 0) -> torch.Tensor:
+             pool: int = 0, v_dim: int = 0) -> torch.Tensor:
     """Causal attention against the cache with score modifiers, all in
     fp32: s = q.k * scale * temp[h]; s = cap*tanh(s/cap);
     s -= r1[h] * ln(1 + r2[h] * (i-j)); softmax whose denominator also
@@ -597,8 +597,13 @@ def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
     i also sees entry c of the pooled caches ``pool_k`` / ``pool_v``
     [Bc, Hkv, Sp, D|Dv] for every block c that ends at or before i - window
     (c < (i - window + 1) // pool), in the same softmax; pooled entries take
-    no distance penalty."""
+    no distance penalty.
+
+    ``vcache`` None: the values are the first ``v_dim`` entries of the key
+    rows (latent attention: one cached latent is key and value)."""
     Hkv, D = kcache.shape[1], kcache.shape[3]
+    if vcache is None:
+        vcache = kcache[..., :v_dim]
     Dv = vcache.shape[3]
     M = q.shape[0]
     B = M // T
@@ -884,3 +889,145 @@ def clamped_glu(gu: torch.Tensor, alpha: float, limit: float) -> torch.Tensor:
     g = gu[..., :i].float().clamp(max=limit)
     u = gu[..., i:].float().clamp(min=-limit, max=limit)
     return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
+
+
+# ---- residual streams, gated delta rule, latent attention (komizen) ----
+
+def hc_read_norm(xs: torch.Tensor, w_in: torch.Tensor, wn: torch.Tensor,
+                 eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """Read of a set of residual streams: xs fp32 [M, S*W] holds S streams
+    of width W side by side; u = sum_s w_in[s] * x_s, returned RMS-normalized
+    times wn [W] (statistics in fp32)."""
+    S = w_in.numel()
+    M = xs.shape[0]
+    x = xs.view(M, S, -1)
+    u = x[:, 0] * w_in[0]
+    for s in range(1, S):
+        u = u + x[:, s] * w_in[s]
+    return rmsnorm_rows(u, wn, eps, out_dtype)
+
+
+def hc_write(xs: torch.Tensor, y: torch.Tensor, mix: torch.Tensor,
+             w_out: torch.Tensor, next_in, next_wn, eps: float,
+             out_dtype: torch.dtype):
+    """Write of a sublayer's result y [M, W] into the streams, all streams at
+    once from the old ones: x_t <- sum_s mix[s, t] x_s + w_out[t] y (xs fp32
+    [M, S*W], in place). With ``next_in`` / ``next_wn`` the read of the next
+    sublayer (``hc_read_norm``) is returned as well."""
+    S = w_out.numel()
+    M = xs.shape[0]
+    old = xs.view(M, S, -1).clone()
+    new = xs.view(M, S, -1)
+    yf = y.float()
+    for t in range(S):
+        acc = old[:, 0] * mix[0, t]
+        for s in range(1, S):
+            acc = acc + old[:, s] * mix[s, t]
+        new[:, t] = acc + w_out[t] * yf
+    if next_in is None:
+        return None
+    return hc_read_norm(xs, next_in, next_wn, eps, out_dtype)
+
+
+def gated_delta_scan(qkv: torch.Tensor, gates: torch.Tensor, b_col0: int,
+                     a_col0: int, a_log: torch.Tensor, dt_bias: torch.Tensor,
+                     state: torch.Tensor, pos: torch.Tensor, T: int, H: int,
+                     KH: int, d: int, dv: int, unit_eps: float, lens=None,
+                     slots=None) -> torch.Tensor:
+    """Gated delta rule, all fp32. qkv fp32 [B*T, 2*KH*d + H*dv] = [q | k |
+    v] (KH query/key heads shared by H/KH value heads each); columns
+    [b_col0, +H) and [a_col0, +H) of ``gates`` hold the raw write-strength
+    and decay projections. Per head h (key head h // (H/KH)), with q, k made
+    unit vectors (x / sqrt(sum x^2 + unit_eps)), q scaled by d^-1/2,
+    beta = sigmoid(b), g = exp(-exp(a_log[h]) softplus(a + dt_bias[h])):
+        S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+    ``state`` fp32 [Bc, H, d, dv] per slot: zero at position 0. Returns o
+    fp32 [B*T, H*dv]."""
+    M = qkv.shape[0]
+    B = M // T
+    out = torch.zeros(M, H * dv, dtype=torch.float32, device=qkv.device)
+    p, ln, sl = _row_index(B, T, pos, lens, slots, qkv.device)
+    hk = torch.arange(H, device=qkv.device) // (H // KH)
+    for b in range(B):
+        n = int(min(ln[b], T))
+        if n <= 0:
+            continue
+        p0, s = int(p[b]), int(sl[b])
+        S = state[s].float().clone() if p0 > 0 else \
+            torch.zeros(H, d, dv, dtype=torch.float32, device=qkv.device)
+        rows = slice(b * T, b * T + n)
+        q = qkv[rows, :KH * d].float().view(n, KH, d)
+        k = qkv[rows, KH * d:2 * KH * d].float().view(n, KH, d)
+        v = qkv[rows, 2 * KH * d:].float().view(n, H, dv)
+        q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + unit_eps) * d ** -0.5
+        k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + unit_eps)
+        q, k = q[:, hk], k[:, hk]                              # [n, H, d]
+        beta = torch.sigmoid(gates[rows, b_col0:b_col0 + H].float())
+        g = torch.exp(-torch.exp(a_log.float()) * torch.nn.functional.softplus(
+            gates[rows, a_col0:a_col0 + H].float() + dt_bias.float(),
+            threshold=30.0))
+        for t in range(n):
+            S = g[t].view(H, 1, 1) * S
+            u = beta[t].view(H, 1) * (
+                v[t] - torch.einsum("hij,hi->hj", S, k[t]))
+            S = S + k[t].unsqueeze(-1) * u.unsqueeze(1)
+            out[b * T + t] = torch.einsum("hij,hi->hj", S, q[t]).reshape(-1)
+        state[s] = S
+    return out
+
+
+def latent_append(src: torch.Tensor, col0: int, wn: torch.Tensor, eps: float,
+                  R: int, rot_freq: torch.Tensor, kcache: torch.Tensor,
+                  pos: torch.Tensor, T: int, lens=None, slots=None) -> None:
+    """Append the shared key/value latent of latent attention to the cache.
+    Columns [col0, col0+R) of src [B*T, ld] are RMS-normalized times wn [R];
+    the rd = 2*len(rot_freq) columns after them turn by position (interleaved
+    pairs, angle = position * rot_freq[i], fp32). The cache row [normed
+    latent | turned key part] goes to kcache [Bc, 1, Smax, R+rd] at position
+    pos[b]+t of row slots[b]; padding tokens are not appended."""
+    M = src.shape[0]
+    B = M // T
+    rd = 2 * rot_freq.numel()
+    c = rmsnorm_rows(src[:, col0:col0 + R], wn, eps, torch.float32)
+    p, ln, sl = _row_index(B, T, pos, lens, slots, src.device)
+    tpos = (p.view(B, 1) + torch.arange(T, device=src.device)
+            ).reshape(M).to(torch.float32)
+    ang = tpos.view(M, 1) * rot_freq.float().view(1, -1)
+    kr = rotate_pairs(src[:, col0 + R:col0 + R + rd].float().view(M, 1, rd),
+                      ang).view(M, rd)
+    row = torch.cat([c, kr], dim=1).to(kcache.dtype)
+    for b in range(B):
+        n = int(min(ln[b], T))
+        if n <= 0:
+            continue
+        p0, s = int(p[b]), int(sl[b])
+        kcache[s, 0, p0:p0 + n] = row[b * T:b * T + n]
+
+
+def latent_q_pack(q: torch.Tensor, qabs: torch.Tensor,
+                  rot_freq: torch.Tensor, pos: torch.Tensor, T: int, H: int,
+                  d: int) -> torch.Tensor:
+    """Queries of latent attention in the cache's layout. q [B*T, H*(d+rd)]
+    holds per head d plain and rd turning dimensions; qabs [H, B*T, R] the
+    plain part already carried into the latent space. Returns [B*T,
+    H*(R+rd)] = per head [qabs | turned part] (angles as in
+    ``latent_append``)."""
+    M = q.shape[0]
+    B = M // T
+    rd = 2 * rot_freq.numel()
+    R = qabs.shape[2]
+    tpos = (pos.to(torch.int64).view(B, 1)
+            + torch.arange(T, device=q.device)).reshape(M).to(torch.float32)
+    ang = tpos.view(M, 1) * rot_freq.float().view(1, -1)
+    qr = rotate_pairs(q.view(M, H, d + rd)[..., d:].float(), ang)
+    out = torch.cat([qabs.transpose(0, 1).float(), qr], dim=-1)
+    return out.reshape(M, H * (R + rd)).to(q.dtype)
+
+
+def moe_up_act(x: torch.Tensor, w: torch.Tensor, we: torch.Tensor
+               ) -> torch.Tensor:
+    """Ungated experts' first half: x [M, K], stacked w [E, I, K], we [M, E]
+    -> act [E, M, I] = relu(x w_e^T)^2 in bf16 (experts nobody chose may
+    hold anything; ``moe_down`` never reads them)."""
+    z = torch.einsum("mk,eik->emi", x.float(), w.float())
+    return (torch.relu(z) ** 2).to(torch.bfloat16)

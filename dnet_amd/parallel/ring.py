@@ -139,7 +139,11 @@ class RingExecutor:
         self.kvs = [self.model.make_kv_cache(mb_size, smax)
                     for _ in range(mb_count)]
         self.sampler = Sampler(decoding or DecodingConfig())
-        H = cfg.hidden_size
+        # width of one row of the residual as the windows take and return it
+        # (several residual streams side by side for families that keep
+        # more than one)
+        H = self.hidden_width = int(getattr(self.model, "hidden_width",
+                                            cfg.hidden_size))
         # static buffers (recv targets / graph inputs)
         # (residual-stream dtype is the model's: bf16, or fp32 for
         # families that keep the residual in 32-bit)
@@ -164,7 +168,7 @@ class RingExecutor:
         self.compress_ratio = compress_ratio if 0.0 < compress_ratio < 1.0 else 0.0
         if self.compress_ratio:
             from ..compression import keep_count
-            k = keep_count(cfg.hidden_size, self.compress_ratio)
+            k = keep_count(H, self.compress_ratio)
             self._cidx = [torch.zeros(k, dtype=torch.int32, device=self.device)
                           for _ in range(mb_count)]
             self._cpacked = [torch.zeros(mb_size, k, dtype=torch.bfloat16,
@@ -221,7 +225,7 @@ class RingExecutor:
         self.ring.recv(self._cpacked[mb])
         self.hbuf[mb].copy_(
             column_unsparsify(self._cpacked[mb], self._cidx[mb],
-                              self.cfg.hidden_size))
+                              self.hidden_width))
 
     # ------------- one-rank step bodies (graph-capturable) -------------
 
@@ -321,7 +325,7 @@ class RingExecutor:
         every rank."""
         M, B, T = tokens.shape
         assert M == self.mb_count and B == self.mb_size
-        H = self.cfg.hidden_size
+        H = self.hidden_width
         tok_reqs = []
         first_tokens = torch.zeros(M, B, dtype=torch.int64, device=self.device)
         last_r = self.rounds - 1
@@ -510,7 +514,7 @@ class RingExecutor:
             "prompt longer than the KV capacity"
         groups = ([list(range(n))] if self.model.ragged_prefill
                   else [[i] for i in range(n)])
-        H = self.cfg.hidden_size
+        H = self.hidden_width
         kv = self.kvs[0]
         picked: list = [[None] * len(w) for w in want]
         for grp in groups:
@@ -597,7 +601,7 @@ class RingExecutor:
             return
         assert self.mb_count == 1
         self.kvs[0].grow(n)
-        self.hbuf = [torch.zeros(n, self.cfg.hidden_size,
+        self.hbuf = [torch.zeros(n, self.hidden_width,
                                  dtype=self.model.act_dtype,
                                  device=self.device)]
         tb = torch.zeros(n, dtype=torch.int64, device=self.device)

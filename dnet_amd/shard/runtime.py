@@ -264,16 +264,19 @@ class ShardRuntime:
         from ..utils import repack as rp
         model_id = req.model_name or req.model_path
         need_api = ex.is_first or ex.is_last
+        # stored layers behind this shard's layer runs (a looped span of
+        # layers runs several times on one set of tensors)
+        stored = ex.cfg.stored_layers(ex.my_layers)
         if self.settings.storage.repack_on_load:
-            sd = rp.load_repacked(model_id, ex.my_layers, include_api=need_api)
+            sd = rp.load_repacked(model_id, stored, include_api=need_api)
             if sd is not None:
                 log.info("repack fastpath: loaded %d tensors from %s",
-                         len(sd), rp.repack_dir_for(model_id, ex.my_layers))
+                         len(sd), rp.repack_dir_for(model_id, stored))
                 ex.model.load_state_dict(sd)
                 return
         meta = get_model_metadata(req.model_path)
         names: list[str] = []
-        for lid in ex.my_layers:
+        for lid in stored:
             names += meta.layers.get(lid, [])
         if ex.is_first:
             names += meta.embed
@@ -285,7 +288,7 @@ class ShardRuntime:
                 # repack for free from the just-loaded tensors: the next
                 # load of this assignment skips the full-safetensors parse
                 rp.ensure_repacked_for_layers(req.model_path, model_id,
-                                              ex.my_layers,
+                                              stored,
                                               include_api=need_api, sd=sd)
             except Exception:
                 log.exception("repack write failed (non-fatal)")
