@@ -100,6 +100,10 @@ struct ModParams {
   const void* pk;      // pooled caches (same dtype as the cache) or null
   const void* pv;
   int T, Bc, Hq, Hkv, Smax, D, DV, QT, window, pool, Sp;
+  // VS: elements between consecutive value rows of the cache. vshare: the
+  // values are the first DV entries of the key rows (latent attention), the
+  // value pointer is the key pointer and VS = D.
+  int VS, vshare;
   float scale, softcap;
 };
 
@@ -165,13 +169,17 @@ __global__ __launch_bounds__(256) void attn_mod_rows(
   const int nt = min(P.QT, n - t0);
   const int rows = nt * Gb;
   const int D = P.D, DV = P.DV;
-  const int PK = pitch_of(D, sizeof(T)), PV = pitch_of(DV, sizeof(T));
+  const bool vshare = P.vshare != 0;
+  const int PK = pitch_of(D, sizeof(T));
+  const int PV = vshare ? PK : pitch_of(DV, sizeof(T));
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
 
   extern __shared__ __attribute__((aligned(16))) char smem[];
   T* k_lds = reinterpret_cast<T*>(smem);                 // [64][PK]
-  T* v_lds = k_lds + kChunkR * PK;                       // [64][PV]
-  T* q_lds = v_lds + kChunkR * PV;                       // [16][PK]
+  // shared values: the staged key rows are read again as value rows
+  T* v_lds = vshare ? k_lds : k_lds + kChunkR * PK;      // [64][PV]
+  T* q_lds = k_lds + kChunkR * PK +
+             (vshare ? 0 : kChunkR * PV);                // [16][PK]
   float* p_lds = reinterpret_cast<float*>(q_lds + kRowsMax * PK);  // [4][64]
 
   const int64_t qstride = (int64_t)P.Hq * D;
@@ -205,7 +213,8 @@ __global__ __launch_bounds__(256) void attn_mod_rows(
   const int kv_begin =
       P.window > 0 ? max(0, p0 + t0 - P.window + 1) : 0;
   const int64_t kbase = ((int64_t)slot * P.Hkv + hkv) * P.Smax * D;
-  const int64_t vbase = ((int64_t)slot * P.Hkv + hkv) * P.Smax * DV;
+  const int64_t vbase = ((int64_t)slot * P.Hkv + hkv) * P.Smax * P.VS;
+  const int VS = P.VS;
 
   // chunk list: pooled entries first, then the token range
   const int np_max = pool_count(p0 + t0 + nt - 1, P.window, P.pool, P.Sp);
@@ -222,7 +231,7 @@ __global__ __launch_bounds__(256) void attn_mod_rows(
     const T* kc = pooled ? reinterpret_cast<const T*>(P.pk) + pkbase
                          : kc_tok + kbase;
     const T* vc = pooled ? reinterpret_cast<const T*>(P.pv) + pvbase
-                         : vc_tok + vbase;
+                         : vc_tok + vbase;   // (pooled entries: VS == DV)
     __syncthreads();          // previous chunk consumed (and q staged)
     if (VEC) {
       const int dk = D / EV, dvv = DV / EV;
@@ -231,22 +240,24 @@ __global__ __launch_bounds__(256) void attn_mod_rows(
         stage16(&k_lds[r * PK + e], &kc[(int64_t)(s0 + r) * D + e],
                 r < valid);
       }
-      for (int idx = threadIdx.x; idx < kChunkR * dvv; idx += blockDim.x) {
-        const int r = idx / dvv, e = (idx % dvv) * EV;
-        stage16(&v_lds[r * PV + e], &vc[(int64_t)(s0 + r) * DV + e],
-                r < valid);
-      }
+      if (!vshare)
+        for (int idx = threadIdx.x; idx < kChunkR * dvv; idx += blockDim.x) {
+          const int r = idx / dvv, e = (idx % dvv) * EV;
+          stage16(&v_lds[r * PV + e], &vc[(int64_t)(s0 + r) * VS + e],
+                  r < valid);
+        }
     } else {
       for (int idx = threadIdx.x; idx < kChunkR * D; idx += blockDim.x) {
         const int r = idx / D, e = idx % D;
         k_lds[r * PK + e] =
             r < valid ? kc[(int64_t)(s0 + r) * D + e] : (T)0;
       }
-      for (int idx = threadIdx.x; idx < kChunkR * DV; idx += blockDim.x) {
-        const int r = idx / DV, e = idx % DV;
-        v_lds[r * PV + e] =
-            r < valid ? vc[(int64_t)(s0 + r) * DV + e] : (T)0;
-      }
+      if (!vshare)
+        for (int idx = threadIdx.x; idx < kChunkR * DV; idx += blockDim.x) {
+          const int r = idx / DV, e = idx % DV;
+          v_lds[r * PV + e] =
+              r < valid ? vc[(int64_t)(s0 + r) * VS + e] : (T)0;
+        }
     }
     __syncthreads();
 #pragma unroll
@@ -421,7 +432,8 @@ __global__ __launch_bounds__(256) void attn_mod_mfma(
   const int qrow = min(qt + row, n - 1);
   const short* qp = q + ((int64_t)b * P.T + qrow) * P.Hq * D + (int64_t)h * D;
   const short* kp = kc + ((int64_t)slot * P.Hkv + hk) * P.Smax * D;
-  const short* vp = vc + ((int64_t)slot * P.Hkv + hk) * P.Smax * DV;
+  const int VS = P.VS;
+  const short* vp = vc + ((int64_t)slot * P.Hkv + hk) * P.Smax * VS;
 
   bf16x8 qf[DC];
 #pragma unroll
@@ -482,8 +494,8 @@ __global__ __launch_bounds__(256) void attn_mod_mfma(
       const int sg = min(s0 + sr, Sdim - 1);
       short v0 = 0, v1 = 0;
       if (dc < DV) {              // DV is even (multiple of 8)
-        v0 = vp[(int64_t)sg * DV + dc];
-        v1 = vp[(int64_t)sg * DV + dc + 1];
+        v0 = vp[(int64_t)sg * VS + dc];
+        v1 = vp[(int64_t)sg * VS + dc + 1];
       }
       vt_lds[dc * SP + sr] = v0;
       vt_lds[(dc + 1) * SP + sr] = v1;
@@ -596,7 +608,8 @@ static const int* opt_i32(const c10::optional<torch::Tensor>& t, int64_t n,
   return t->data_ptr<int>();
 }
 
-void attn_mod(torch::Tensor q, torch::Tensor kcache, torch::Tensor vcache,
+void attn_mod(torch::Tensor q, torch::Tensor kcache,
+              c10::optional<torch::Tensor> vcache_opt,
               torch::Tensor pos, c10::optional<torch::Tensor> lens,
               c10::optional<torch::Tensor> slots, torch::Tensor out,
               int64_t T, double scale, c10::optional<torch::Tensor> temp,
@@ -605,13 +618,20 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache, torch::Tensor vcache,
               c10::optional<torch::Tensor> sinks, int64_t window,
               c10::optional<torch::Tensor> partials, int64_t splits,
               c10::optional<torch::Tensor> pool_k,
-              c10::optional<torch::Tensor> pool_v, int64_t pool) {
+              c10::optional<torch::Tensor> pool_v, int64_t pool,
+              int64_t v_dim) {
+  // no value cache: values = the first v_dim entries of the key rows
+  const bool vshare = !vcache_opt.has_value();
+  const torch::Tensor& vcache = vshare ? kcache : *vcache_opt;
   DNET_CHECK(kcache.dim() == 4 && vcache.dim() == 4 &&
                  kcache.is_contiguous() && vcache.is_contiguous(), "cache");
   const int Bc = kcache.size(0), Hkv = kcache.size(1), Smax = kcache.size(2);
-  const int D = kcache.size(3), DV = vcache.size(3);
+  const int D = kcache.size(3);
+  const int DV = vshare ? (int)v_dim : (int)vcache.size(3);
   DNET_CHECK(vcache.size(0) == Bc && vcache.size(1) == Hkv &&
                  vcache.size(2) == Smax, "k/v cache shapes differ");
+  DNET_CHECK(!vshare || (DV >= 1 && DV <= D && pool == 0),
+             "shared values: 1 <= v_dim <= key size, no pooled blocks");
   const int64_t M = q.size(0);
   DNET_CHECK(T > 0 && M % T == 0, "rows = B*T");
   const int64_t B = M / T;
@@ -638,6 +658,7 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache, torch::Tensor vcache,
   P.sinks = opt_f32(sinks, Hq, "sinks fp32 [Hq]");
   P.T = (int)T; P.Bc = Bc; P.Hq = Hq; P.Hkv = Hkv; P.Smax = Smax;
   P.D = D; P.DV = DV; P.window = (int)window;
+  P.VS = vshare ? D : DV; P.vshare = vshare ? 1 : 0;
   P.scale = (float)scale; P.softcap = (float)softcap;
   P.pk = P.pv = nullptr;
   P.pool = 0; P.Sp = 0;
@@ -666,7 +687,7 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache, torch::Tensor vcache,
   DNET_CHECK(f32 || q.scalar_type() == torch::kBFloat16, "bf16 or fp32");
   const int es = f32 ? 4 : 2;
   const int PK = pitch_of(D, es), PV = pitch_of(DV, es);
-  const size_t lds = (size_t)es * (kChunkR * PK + kChunkR * PV +
+  const size_t lds = (size_t)es * (kChunkR * PK + (vshare ? 0 : kChunkR * PV) +
                                    kRowsMax * PK) + sizeof(float) * 4 * kChunkR;
   DNET_CHECK(lds <= 160 * 1024, "attn_mod: head sizes exceed LDS");
   const dim3 grid((unsigned)((T + P.QT - 1) / P.QT), (unsigned)(Hkv * GS),

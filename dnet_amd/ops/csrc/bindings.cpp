@@ -118,7 +118,8 @@ void delta_scan(torch::Tensor src, int64_t r0, int64_t k0, int64_t v0,
                 torch::Tensor pos, c10::optional<torch::Tensor> lens,
                 c10::optional<torch::Tensor> slots, int64_t T, int64_t H,
                 int64_t d, double decay_scale, double unit_eps);
-void attn_mod(torch::Tensor q, torch::Tensor kcache, torch::Tensor vcache,
+void attn_mod(torch::Tensor q, torch::Tensor kcache,
+              c10::optional<torch::Tensor> vcache,
               torch::Tensor pos, c10::optional<torch::Tensor> lens,
               c10::optional<torch::Tensor> slots, torch::Tensor out,
               int64_t T, double scale, c10::optional<torch::Tensor> temp,
@@ -127,7 +128,32 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache, torch::Tensor vcache,
               c10::optional<torch::Tensor> sinks, int64_t window,
               c10::optional<torch::Tensor> partials, int64_t splits,
               c10::optional<torch::Tensor> pool_k,
-              c10::optional<torch::Tensor> pool_v, int64_t pool);
+              c10::optional<torch::Tensor> pool_v, int64_t pool,
+              int64_t v_dim);
+void hc_write_read(torch::Tensor xs, c10::optional<torch::Tensor> y,
+                   c10::optional<torch::Tensor> mix,
+                   c10::optional<torch::Tensor> w_out,
+                   c10::optional<torch::Tensor> next_in,
+                   c10::optional<torch::Tensor> next_wn,
+                   c10::optional<torch::Tensor> out, double eps);
+void gated_delta_scan(torch::Tensor qkv, torch::Tensor gates, int64_t b_col0,
+                      int64_t a_col0, torch::Tensor a_log,
+                      torch::Tensor dt_bias, torch::Tensor state,
+                      torch::Tensor o, torch::Tensor pos,
+                      c10::optional<torch::Tensor> lens,
+                      c10::optional<torch::Tensor> slots, int64_t T,
+                      int64_t H, int64_t KH, int64_t d, int64_t dv,
+                      double unit_eps);
+void latent_append(torch::Tensor src, int64_t col0, torch::Tensor wn,
+                   double eps, int64_t R, torch::Tensor rot_freq,
+                   torch::Tensor kcache, torch::Tensor pos,
+                   c10::optional<torch::Tensor> lens,
+                   c10::optional<torch::Tensor> slots, int64_t T);
+void latent_q_pack(torch::Tensor q, torch::Tensor qabs, torch::Tensor rot_freq,
+                   torch::Tensor pos, torch::Tensor out, int64_t T, int64_t H,
+                   int64_t d);
+void moe_up_act(torch::Tensor x, torch::Tensor w, torch::Tensor we,
+                torch::Tensor act);
 }  // namespace dnet
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -208,4 +234,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("ssd_scan", &dnet::ssd_scan,
         "selective state-space recurrence (scalar decay per head)");
   m.def("delta_scan", &dnet::delta_scan, "generalized delta-rule recurrence");
+  m.def("hc_write_read", &dnet::hc_write_read,
+        "residual streams: write a sublayer's result, read the next input");
+  m.def("gated_delta_scan", &dnet::gated_delta_scan,
+        "gated delta-rule recurrence");
+  m.def("latent_append", &dnet::latent_append,
+        "latent attention: norm + rotation + cache append of the shared row");
+  m.def("latent_q_pack", &dnet::latent_q_pack,
+        "latent attention: queries in the cache row's layout");
+  m.def("moe_up_act", &dnet::moe_up_act,
+        "grouped ungated expert up projection + squared ReLU");
 }

@@ -204,6 +204,48 @@ __global__ __launch_bounds__(256, M <= 8 ? 4 : 2) void moe_gateup_kernel(
   }
 }
 
+// Ungated experts (up -> squared ReLU -> down): act[e,m,i] =
+// relu(x[m,:] . Wu[e,i,:])^2 with Wu the stacked up weights [E, I, K] (bf16).
+// Same layout as moe_gateup_kernel's bf16 branch with one weight row per
+// wave; experts nobody in the tile chose are skipped.
+template <int M>
+__global__ __launch_bounds__(256, M <= 8 ? 4 : 2) void moe_up_act_kernel(
+    const short* __restrict__ x, const short* __restrict__ w,
+    const float* __restrict__ we, short* __restrict__ act, const int K,
+    const int I, const int E, const int Mtot, const int m0) {
+  const int e = blockIdx.z;
+  if (!expert_routed<M>(we, E, e, m0)) return;
+  const int wid = threadIdx.x / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int i = blockIdx.x * kMoeWaves + wid;
+  if (i >= I) return;
+  const short8* wu =
+      reinterpret_cast<const short8*>(w + ((int64_t)e * I + i) * K);
+  float au[M];
+#pragma unroll
+  for (int m = 0; m < M; ++m) au[m] = 0.f;
+  const int vecs = K / 8;
+  for (int v = lane; v < vecs; v += kWave) {
+    const short8 uv = wu[v];
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      const short8 xv =
+          reinterpret_cast<const short8*>(x + (int64_t)(m0 + m) * K)[v];
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        au[m] = fmaf(bits2f(uv.x[j]), bits2f(xv.x[j]), au[m]);
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+    float u = wave_reduce_sum(au[m]);
+    if (lane == 0) {
+      u = fmaxf(u, 0.f);
+      act[((int64_t)e * Mtot + m0 + m) * I + i] = f2bits(u * u);
+    }
+  }
+}
+
 template <int M, int QMODE, bool PACKED>
 __global__ __launch_bounds__(256, 4) void moe_down_kernel(
     const short* __restrict__ act, const void* __restrict__ w,
@@ -411,6 +453,38 @@ void moe_gateup(torch::Tensor x, torch::Tensor w,
       } else {
         with_glu(std::integral_constant<int, 0>{}, std::false_type{});
       }
+    });
+    m0 += mt;
+  }
+}
+
+void moe_up_act(torch::Tensor x, torch::Tensor w, torch::Tensor we,
+                torch::Tensor act) {
+  const int64_t M = x.size(0), K = x.size(1);
+  const int64_t E = w.size(0), I = w.size(1);
+  DNET_CHECK(x.scalar_type() == torch::kBFloat16 &&
+                 w.scalar_type() == torch::kBFloat16 &&
+                 act.scalar_type() == torch::kBFloat16 &&
+                 we.scalar_type() == torch::kFloat, "moe_up_act dtypes");
+  DNET_CHECK(w.dim() == 3 && w.size(2) == K && act.size(0) == E &&
+                 act.size(1) == M && act.size(2) == I, "moe_up_act shape");
+  DNET_CHECK(we.size(0) == M && we.size(1) == E, "we shape");
+  DNET_CHECK(x.is_contiguous() && w.is_contiguous() && we.is_contiguous() &&
+                 act.is_contiguous(), "contig");
+  DNET_CHECK(K % 8 == 0, "K align");
+  auto stream = current_stream();
+  const dim3 grid(cdiv((int)I, kMoeWaves), 1, (unsigned)E);
+  int64_t m0 = 0;
+  while (m0 < M) {
+    const int mt = moe_mtile(M - m0, false, 8);
+    moe_dispatch_m(mt, [&](auto mc) {
+      constexpr int MV = decltype(mc)::value;
+      hipLaunchKernelGGL((moe_up_act_kernel<MV>), grid,
+                         dim3(kMoeWaves * kWave), 0, stream,
+                         (const short*)x.data_ptr(),
+                         (const short*)w.data_ptr(),
+                         (const float*)we.data_ptr(), (short*)act.data_ptr(),
+                         (int)K, (int)I, (int)E, (int)M, (int)m0);
     });
     m0 += mt;
   }

@@ -1,5 +1,5 @@
 // Per-slot sequence state beside the KV cache (gfx950): pooled-block caches,
-// short causal convolutions and two linear recurrences.
+// short causal convolutions and three linear recurrences.
 //
 //   kv_pool_update    block means of the cached keys/values for the blocks a
 //                     step completes (read by attn_mod's pooled entries)
@@ -7,6 +7,7 @@
 //                     inputs of every slot are its state
 //   ssd_scan          S <- exp(-exp(A_h) dt) S + dt B x^T ; y = S^T C + D x
 //   delta_scan        S <- diag(w) S - (a u)(u^T S) + k v^T ; o = S^T r
+//   gated_delta_scan  S <- g S ; S <- S + k (beta (v - S^T k))^T ; o = S^T q
 //
 // Geometry is the cache's: token (b,t) = row b*T+t sits at position pos[b]+t
 // of slot slots[b] (default b); tokens t >= lens[b] are padding. Every state
@@ -15,7 +16,7 @@
 // Decays, step sizes, gates and states are fp32 whatever the activation
 // dtype ("short" stands for bf16 bits).
 //
-// The two scans share one layout: a workgroup owns one head (or a slice of
+// The scans share one layout: a workgroup owns one head (or a slice of
 // its value columns) of one batch row and walks the tokens in order. The
 // state matrix [rows x columns] is spread as: thread (column j, slice s)
 // keeps rows [R s, R s + R) of column j in registers (R = 32, 16 or 8); the slices of a
@@ -488,6 +489,148 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(
   }
 }
 
+// ---- gated delta rule --------------------------------------------------------
+// S <- g S ; u = beta (v - S^T k) ; S <- S + k u^T ; o = S^T q, state [d x dv]
+// per value head, q/k heads shared by groups of value heads. grid (H * column
+// tiles, B), block = JB value columns x NS key slices. LDS per token of a
+// chunk: unit q (times d^-1/2), unit k [DP each], v [JB], beta, g. q, k, v
+// come from the convolution's fp32 output; the raw write-strength and decay
+// projections from columns of `gates` (activation dtype).
+template <typename T, int R>
+__global__ __launch_bounds__(256) void gated_delta_scan_kernel(
+    const float* __restrict__ qkv, const T* __restrict__ gates,
+    const int64_t gld, const int b0, const int a0,
+    const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+    float* __restrict__ state, float* __restrict__ o, const Geo g,
+    const int H, const int KH, const int d, const int dv, const int JB,
+    const int NS, const int TC, const float unit_eps) {
+  const int ntile = (dv + JB - 1) / JB;
+  const int h = blockIdx.x / ntile;
+  const int j0 = (blockIdx.x % ntile) * JB;
+  const int b = blockIdx.y;
+  int p0, n, slot;
+  if (!row_geo(g, b, p0, n, slot)) return;
+  const int kh = h / (H / KH);
+  const int C = 2 * KH * d + H * dv;
+  const int DR = NS * R;                    // key rows incl. padding
+  const int DP = NS * (R + 4);              // LDS pitch of one token
+  const int jl = threadIdx.x / NS, sl = threadIdx.x % NS;
+  const int j = j0 + jl;
+  const bool col_ok = j < dv;
+  const int wid = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const int nw = (blockDim.x + kWave - 1) / kWave;
+
+  extern __shared__ __attribute__((aligned(16))) float sm[];
+  float* sQ = sm;                               // [TC][DP]
+  float* sK = sQ + TC * DP;
+  float* sV = sK + TC * DP;                     // [TC][JB]
+  float* sBeta = sV + TC * JB;                  // [TC]
+  float* sG = sBeta + TC;                       // [TC]
+
+  float S[R];
+  float* sp = state + (((int64_t)slot * H + h) * d) * dv;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int row = sl * R + r;
+    S[r] = (p0 > 0 && col_ok && row < d) ? sp[(int64_t)row * dv + j] : 0.f;
+  }
+  const float a_h = expf(a_log[h]), bias_h = dt_bias[h];
+  const float qscale = 1.0f / sqrtf((float)d);
+
+  for (int t0 = 0; t0 < n; t0 += TC) {
+    const int tc = min(TC, n - t0);
+    __syncthreads();                            // previous chunk consumed
+    for (int idx = threadIdx.x; idx < tc * DR; idx += blockDim.x) {
+      const int tt = idx / DR, i = idx % DR;
+      const float* sr = qkv + ((int64_t)b * g.T + t0 + tt) * C;
+      const int at = tt * DP + padded<R>(i);
+      sQ[at] = i < d ? sr[kh * d + i] : 0.f;
+      sK[at] = i < d ? sr[KH * d + kh * d + i] : 0.f;
+    }
+    for (int idx = threadIdx.x; idx < tc * JB; idx += blockDim.x) {
+      const int tt = idx / JB, c = idx % JB;
+      sV[idx] = (j0 + c < dv)
+                    ? qkv[((int64_t)b * g.T + t0 + tt) * C + 2 * KH * d +
+                          h * dv + j0 + c]
+                    : 0.f;
+    }
+    for (int tt = threadIdx.x; tt < tc; tt += blockDim.x) {
+      const T* gr = gates + ((int64_t)b * g.T + t0 + tt) * gld;
+      sBeta[tt] = sigmoid_a(lds<T>(gr + b0 + h));
+      sG[tt] = expf(-a_h * softplus_a(lds<T>(gr + a0 + h) + bias_h));
+    }
+    __syncthreads();
+    // unit vectors: x / sqrt(sum x^2 + eps), q also times d^-1/2
+    for (int tt = wid; tt < tc; tt += nw) {
+      float sq = 0.f, sk = 0.f;
+      for (int i = lane; i < d; i += kWave) {
+        const float qv = sQ[tt * DP + padded<R>(i)];
+        const float kv = sK[tt * DP + padded<R>(i)];
+        sq = fmaf(qv, qv, sq);
+        sk = fmaf(kv, kv, sk);
+      }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        sq += __shfl_xor(sq, off, 64);
+        sk += __shfl_xor(sk, off, 64);
+      }
+      const float rq = qscale / sqrtf(sq + unit_eps);
+      const float rk = 1.0f / sqrtf(sk + unit_eps);
+      for (int i = lane; i < d; i += kWave) {
+        sQ[tt * DP + padded<R>(i)] *= rq;
+        sK[tt * DP + padded<R>(i)] *= rk;
+      }
+    }
+    __syncthreads();
+    for (int tt = 0; tt < tc; ++tt) {
+      const int base = tt * DP + sl * (R + 4);
+      const float4* kp = reinterpret_cast<const float4*>(sK + base);
+      const float4* qp = reinterpret_cast<const float4*>(sQ + base);
+      const float gt = sG[tt];
+      float ks = 0.f;                           // (S^T k)_j over my rows
+#pragma unroll
+      for (int r4 = 0; r4 < R / 4; ++r4) {
+        const float4 kv = kp[r4];
+        S[4 * r4 + 0] *= gt;
+        S[4 * r4 + 1] *= gt;
+        S[4 * r4 + 2] *= gt;
+        S[4 * r4 + 3] *= gt;
+        ks = fmaf(kv.x, S[4 * r4 + 0], ks);
+        ks = fmaf(kv.y, S[4 * r4 + 1], ks);
+        ks = fmaf(kv.z, S[4 * r4 + 2], ks);
+        ks = fmaf(kv.w, S[4 * r4 + 3], ks);
+      }
+      for (int off = NS >> 1; off > 0; off >>= 1)
+        ks += __shfl_xor(ks, off, 64);
+      const float uj = sBeta[tt] * (sV[tt * JB + jl] - ks);
+      float acc = 0.f;
+#pragma unroll
+      for (int r4 = 0; r4 < R / 4; ++r4) {
+        const float4 kv = kp[r4], qv = qp[r4];
+        S[4 * r4 + 0] = fmaf(kv.x, uj, S[4 * r4 + 0]);
+        S[4 * r4 + 1] = fmaf(kv.y, uj, S[4 * r4 + 1]);
+        S[4 * r4 + 2] = fmaf(kv.z, uj, S[4 * r4 + 2]);
+        S[4 * r4 + 3] = fmaf(kv.w, uj, S[4 * r4 + 3]);
+        acc = fmaf(S[4 * r4 + 0], qv.x, acc);
+        acc = fmaf(S[4 * r4 + 1], qv.y, acc);
+        acc = fmaf(S[4 * r4 + 2], qv.z, acc);
+        acc = fmaf(S[4 * r4 + 3], qv.w, acc);
+      }
+      for (int off = NS >> 1; off > 0; off >>= 1)
+        acc += __shfl_xor(acc, off, 64);
+      if (sl == 0 && col_ok)
+        o[((int64_t)b * g.T + t0 + tt) * (int64_t)(H * dv) + h * dv + j] = acc;
+    }
+  }
+  if (col_ok) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int row = sl * R + r;
+      if (row < d) sp[(int64_t)row * dv + j] = S[r];
+    }
+  }
+}
+
 bool is_bf16(const torch::Tensor& t) { return t.scalar_type() == torch::kBFloat16; }
 bool is_f32(const torch::Tensor& t) { return t.scalar_type() == torch::kFloat32; }
 
@@ -740,6 +883,64 @@ void delta_scan(torch::Tensor src, int64_t r0, int64_t k0, int64_t v0,
   else DNET_CHECK(false, "delta_scan: dtype");
 #undef DS_R
 #undef DS
+}
+
+void gated_delta_scan(torch::Tensor qkv, torch::Tensor gates, int64_t b_col0,
+                      int64_t a_col0, torch::Tensor a_log,
+                      torch::Tensor dt_bias, torch::Tensor state,
+                      torch::Tensor o, torch::Tensor pos,
+                      c10::optional<torch::Tensor> lens,
+                      c10::optional<torch::Tensor> slots, int64_t T,
+                      int64_t H, int64_t KH, int64_t d, int64_t dv,
+                      double unit_eps) {
+  const int64_t M = qkv.size(0);
+  DNET_CHECK(T > 0 && M % T == 0, "rows = B*T");
+  const int64_t B = M / T;
+  DNET_CHECK(H > 0 && KH > 0 && H % KH == 0 && d > 0 && d <= 256 && dv > 0,
+             "heads / key heads / key size <= 256");
+  DNET_CHECK(qkv.dim() == 2 && is_f32(qkv) && qkv.is_contiguous() &&
+                 qkv.size(1) == 2 * KH * d + H * dv, "qkv fp32 [B*T, q|k|v]");
+  DNET_CHECK(gates.dim() == 2 && gates.is_contiguous() &&
+                 gates.size(0) == M, "gates [B*T, ld]");
+  for (int64_t c0 : {b_col0, a_col0})
+    DNET_CHECK(c0 >= 0 && c0 + H <= gates.size(1), "gate columns");
+  DNET_CHECK(is_f32(a_log) && a_log.is_contiguous() && a_log.numel() == H &&
+                 is_f32(dt_bias) && dt_bias.is_contiguous() &&
+                 dt_bias.numel() == H, "per-head fp32 parameters");
+  DNET_CHECK(state.dim() == 4 && is_f32(state) && state.is_contiguous() &&
+                 state.size(1) == H && state.size(2) == d &&
+                 state.size(3) == dv, "state fp32 [Bc, H, d, dv]");
+  DNET_CHECK(is_f32(o) && o.is_contiguous() && o.size(0) == M &&
+                 o.size(1) == H * dv, "o fp32 [B*T, H*dv]");
+  if (M == 0) return;
+  const Geo g = make_geo(pos, lens, slots, B, T, state.size(0));
+  int R, NS, JB;
+  scan_shape((int)d, (int)dv, H * B, 8, R, NS, JB);
+  const int DP = NS * (R + 4);
+  int TC = 32;
+  while (TC > 1 && (size_t)TC * (2 * DP + JB + 2) * 4 > 48 * 1024) TC /= 2;
+  const size_t lds_bytes = (size_t)TC * (2 * DP + JB + 2) * sizeof(float);
+  const dim3 grid((unsigned)(H * ((dv + JB - 1) / JB)), (unsigned)B);
+  auto st = current_stream();
+#define GD(TT, RR)                                                           \
+  hipLaunchKernelGGL((gated_delta_scan_kernel<TT, RR>), grid,                \
+                     dim3(JB * NS), lds_bytes, st, qkv.data_ptr<float>(),    \
+                     (const TT*)gates.data_ptr(), gates.size(1),             \
+                     (int)b_col0, (int)a_col0, a_log.data_ptr<float>(),      \
+                     dt_bias.data_ptr<float>(), state.data_ptr<float>(),     \
+                     o.data_ptr<float>(), g, (int)H, (int)KH, (int)d,        \
+                     (int)dv, JB, NS, TC, (float)unit_eps)
+#define GD_R(TT)                          \
+  do {                                    \
+    if (R == 32) GD(TT, 32);              \
+    else if (R == 16) GD(TT, 16);         \
+    else GD(TT, 8);                       \
+  } while (0)
+  if (is_bf16(gates)) GD_R(short);
+  else if (is_f32(gates)) GD_R(float);
+  else DNET_CHECK(false, "gated_delta_scan: gates dtype");
+#undef GD_R
+#undef GD
 }
 
 }  // namespace dnet

@@ -202,3 +202,75 @@ def forward(cfg, sd, tokens, dtype=torch.float32, layers_out=None):
         x = sum(xs)
     x = norm_centered(x, sd["final.norm"].to(dtype), eps)
     return x @ emb.T
+
+
+def make_checkpoint(cfg, seed=0):
+    """Random bf16 tensors under the checkpoint's names for a config dict;
+    scales keep every branch of comparable size."""
+    g = torch.Generator().manual_seed(seed)
+    W, S = cfg["width"], cfg.get("streams")
+
+    def rn(*shape, std=1.0):
+        return (torch.randn(*shape, generator=g) * std).to(torch.bfloat16)
+
+    def ru(n, lo, hi):
+        return (torch.rand(n, generator=g) * (hi - lo) + lo).to(torch.bfloat16)
+
+    def lin(out, inp):
+        return rn(out, inp, std=inp ** -0.5)
+
+    sd = {"embed": rn(cfg["vocab"], W, std=W ** -0.5),
+          "final.norm": rn(W, std=0.1)}
+    for i, spec in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", spec["mixer"]
+        sd[p + "norm1"] = rn(W, std=0.1)
+        subs = [1] + ([2] if spec.get("mlp") else [])
+        if S:
+            for q in subs:
+                sd[p + f"hc{q}.in"] = ru(S, 0.5, 1.0) / S
+                sd[p + f"hc{q}.out"] = ru(S, 0.3, 1.0)
+                sd[p + f"hc{q}.mix"] = (torch.eye(S) * 0.8 + torch.randn(
+                    S, S, generator=g) * 0.15).to(torch.bfloat16)
+        if spec["type"] == "latent_attention":
+            H, d, rd, dv = m["heads"], m["dim"], m["rot_dim"], m["vdim"]
+            R, QR = m["kv_rank"], m["q_rank"]
+            sd.update({p + "mix.dq": lin(QR, W),
+                       p + "mix.dq.norm": 1 + rn(QR, std=0.1),
+                       p + "mix.uq": lin(H * (d + rd), QR) * 2,
+                       p + "mix.dkv": lin(R + rd, W),
+                       p + "mix.dkv.norm": 1 + rn(R, std=0.1),
+                       p + "mix.uk": lin(H * d, R) * 2,
+                       p + "mix.uv": lin(H * dv, R),
+                       p + "mix.o": lin(W, H * dv)})
+        elif spec["type"] == "delta":
+            H, KH, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            taps = m["conv"]
+            sd.update({p + "mix.q": lin(KH * d, W), p + "mix.k": lin(KH * d, W),
+                       p + "mix.v": lin(H * dv, W), p + "mix.g": lin(H * dv, W),
+                       p + "mix.b": lin(H, W), p + "mix.a": lin(H, W),
+                       p + "mix.q.conv": rn(KH * d, taps, std=0.5),
+                       p + "mix.k.conv": rn(KH * d, taps, std=0.5),
+                       p + "mix.v.conv": rn(H * dv, taps, std=0.5),
+                       p + "mix.A_log": ru(H, -3.0, 0.5),
+                       p + "mix.dt_bias": ru(H, -3.0, 0.0),
+                       p + "mix.norm": 1 + rn(dv, std=0.1),
+                       p + "mix.o": lin(W, H * dv)})
+        else:
+            H, P, N, G = m["heads"], m["vdim"], m["state"], m["groups"]
+            inner, C = H * P, H * P + 2 * G * N
+            sd.update({p + "mix.in": lin(2 * inner + 2 * G * N + H, W),
+                       p + "mix.conv": rn(C, m["conv"], std=0.5),
+                       p + "mix.conv.b": rn(C, std=0.1),
+                       p + "mix.dt_bias": ru(H, -3.0, 0.0),
+                       p + "mix.A_log": ru(H, -1.0, 1.5),
+                       p + "mix.D": rn(H),
+                       p + "mix.norm": 1 + rn(inner, std=0.1),
+                       p + "mix.o": lin(W, inner)})
+        ff = spec.get("mlp")
+        if ff:
+            sd[p + "norm2"] = rn(W, std=0.1)
+            sd[p + "mlp.router"] = lin(ff["router"]["experts"], W) * 3
+            for e in range(ff["router"]["experts"]):
+                sd[p + f"mlp.e{e}.up"] = lin(ff["expert"]["ff"], W)
+                sd[p + f"mlp.e{e}.down"] = lin(W, ff["expert"]["ff"])
+    return sd
