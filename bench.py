@@ -55,7 +55,24 @@ _COMPARE_SIZES = [("2k", 2048, 16, 4, 128, 8192),
 
 def _family_hf(fam, W, H, KV, D, FF, layers, vocab, args):
     """config.json-style description of ``fam`` at the given layer sizes."""
-    from dnet_amd.models.config import gegorax_config, posudra_config
+    from dnet_amd.models.config import (gegorax_config, komizen_config,
+                                        posudra_config)
+    if fam == "komizen":
+        # latent attention (every second layer) with gated delta-rule and
+        # mamba2 layers between; 192 + 64 cached entries per token; 4
+        # residual streams; delta-rule and state-space heads of 64 channels
+        # over the model width as in the gegorax stack; every feed-forward a
+        # mixture of ungated experts whose chosen ones together are as wide
+        # as the dense feed-forward it stands beside
+        E = args.compare_experts or 8
+        top = min(2, E)
+        return komizen_config(
+            W, vocab, "ldlm", layers=layers, heads=H, dim=D, rot_dim=64,
+            vdim=D, kv_rank=192, q_rank=max(256, W // 4),
+            delta_heads=W // 64, delta_kv_heads=max(1, W // 128),
+            delta_dim=64, delta_vdim=64, ssm_heads=W // 64, ssm_vdim=64,
+            ssm_state=128, ssm_groups=max(1, W // 512), conv=4, experts=E,
+            top=top, expert_ff=FF // top, streams=4)
     if fam == "posudra":
         return posudra_config(W, layers, H, KV, D, D, FF, vocab)
     if fam == "gegorax":
@@ -79,13 +96,16 @@ def _family_hf(fam, W, H, KV, D, FF, layers, vocab, args):
 
 
 # family -> the closest existing family it is measured beside
-_COMPARE_WITH = {"posudra": "qwen3", "gegorax": "posudra"}
+_COMPARE_WITH = {"posudra": "qwen3", "gegorax": "posudra",
+                 "komizen": "gegorax"}
 
 
 def compare_family(args, device):
     """Prefill and decode throughput of a family beside the closest existing
     one (posudra: qwen3 — dense, grouped heads, q/k norm; gegorax: posudra —
-    one norm feeding parallel branches, fp32 residual, per-layer sizes) at
+    one norm feeding parallel branches, fp32 residual, per-layer sizes;
+    komizen: gegorax — attention beside state-space and delta-rule layers on
+    an fp32 residual with per-slot recurrent state) at
     equal layer sizes, bf16, random weights. One JSON line; the default
     workload is untouched."""
     new, old = args.compare_family, _COMPARE_WITH[args.compare_family]
@@ -174,14 +194,15 @@ def main():
                     help="GPU-resident layers per rank (0=all; <local layers "
                          "enables host-DRAM weight streaming)")
     ap.add_argument("--compare-family", default="",
-                    choices=["", "posudra", "gegorax"],
+                    choices=["", "posudra", "gegorax", "komizen"],
                     help="instead of the default workload: throughput of "
                          "this family beside its closest existing one at "
                          "equal layer sizes")
     ap.add_argument("--compare-layers", type=int, default=8)
     ap.add_argument("--compare-experts", type=int, default=0,
                     help="gegorax: experts of the mixture feed-forward in "
-                         "every second layer (0 = dense feed-forwards)")
+                         "every second layer (0 = dense feed-forwards); "
+                         "komizen: experts of every layer (0 = 8)")
     ap.add_argument("--compare-prefill-batch", type=int, default=8)
     ap.add_argument("--compare-sizes", default="",
                     help="comma list out of 2k,4k,5k (default: all)")

@@ -430,20 +430,25 @@ class KomizenRingModel(RingModel):
         we = torch.zeros(T, E, dtype=torch.float32, device=u.device)
         we.scatter_(1, idx, val * float(ff["router"]["scale"]))
         I = lw.up_w.shape[1]
-        if (T <= self.DENSE_MOE_MAX_T and self.wdtype == torch.bfloat16
+        if (T * top < E and self.wdtype == torch.bfloat16
                 and W % 8 == 0 and I % 8 == 0):
-            # grouped expert kernels: two launches, unrouted experts skipped
-            # on the device (no host sync: graph-capturable)
+            # few rows, most experts idle: grouped expert kernels, two
+            # launches, unrouted experts skipped on the device (no host
+            # sync: graph-capturable), so only the chosen experts' weights
+            # are read
             act = ops.moe_up_act(u, lw.up_w, we)
             return ops.moe_down(act, lw.down_w, None, None, we, 0, False)
-        out = torch.zeros(T, W, dtype=torch.float32, device=u.device)
         if T <= self.DENSE_MOE_MAX_T:
-            # few rows: every expert on every row, weighted (zero for the
-            # experts a row did not choose); no host sync
-            for e in range(E):
-                a = ops.act_slice(u @ lw.up_w[e].t(), 0, I, "relu_sq")
-                out += we[:, e:e + 1] * (a @ lw.down_w[e].t()).float()
-            return out
+            # a decode batch that reaches most experts anyway: every expert
+            # on every row as two batched products (each expert's weights
+            # read once), weighted with zero for the experts a row did not
+            # choose; no host sync
+            z = torch.bmm(u.unsqueeze(0).expand(E, T, W),
+                          lw.up_w.transpose(1, 2))              # [E, T, I]
+            a = ops.act_slice(z.view(E * T, I), 0, I, "relu_sq")
+            d = torch.bmm(a.view(E, T, I), lw.down_w.transpose(1, 2))
+            return torch.einsum("te,etw->tw", we, d.float())
+        out = torch.zeros(T, W, dtype=torch.float32, device=u.device)
         hit = (we > 0).any(dim=0).tolist()
         for e in range(E):
             if not hit[e]:

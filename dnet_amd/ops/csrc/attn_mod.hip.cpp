@@ -705,6 +705,7 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache,
   do {                                     \
     if (DV <= 64) AM(DCC, 4);              \
     else if (DV <= 128) AM(DCC, 8);        \
+    else if (DV <= 192) AM(DCC, 12);       \
     else AM(DCC, 16);                      \
   } while (0)
     if (D <= 64) AM_V(2);

@@ -204,9 +204,12 @@ def forward(cfg, sd, tokens, dtype=torch.float32, layers_out=None):
     return x @ emb.T
 
 
-def make_checkpoint(cfg, seed=0):
+def make_checkpoint(cfg, seed=0, ff_gain=1.0):
     """Random bf16 tensors under the checkpoint's names for a config dict;
-    scales keep every branch of comparable size."""
+    scales keep every branch of comparable size. ``ff_gain`` scales the
+    experts' output: bfloat16 comparisons use a small one, so that a token
+    whose router sits on a near-tie that rounding flips moves the logits
+    little (input-dependent routing is compared in float32)."""
     g = torch.Generator().manual_seed(seed)
     W, S = cfg["width"], cfg.get("streams")
 
@@ -272,5 +275,5 @@ def make_checkpoint(cfg, seed=0):
             sd[p + "mlp.router"] = lin(ff["router"]["experts"], W) * 3
             for e in range(ff["router"]["experts"]):
                 sd[p + f"mlp.e{e}.up"] = lin(ff["expert"]["ff"], W)
-                sd[p + f"mlp.e{e}.down"] = lin(W, ff["expert"]["ff"])
+                sd[p + f"mlp.e{e}.down"] = lin(W, ff["expert"]["ff"]) * ff_gain
     return sd

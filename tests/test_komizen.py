@@ -1,0 +1,662 @@
+"""Komizen in the framework against the plain oracle (tests/komizen_oracle.py).
+
+Every test builds its own small configuration and random checkpoint, runs it
+through the framework's ops / model / cache / executor (and, for generation,
+the shard runtime's slot scheduler and the trace replay CLI) and compares with
+the oracle, which is written from the equations, runs whole sequences without
+any cache and shares no code with dnet_amd. Tests run on the CPU reference-op
+path and, marked ``gpu``, on the HIP kernels.
+"""
+import copy
+import json
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+import torch
+
+import komizen_oracle as O
+from dnet_amd.models import ModelConfig
+from dnet_amd.models.config import komizen_config
+from dnet_amd.parallel.ring import RingExecutor
+
+DEVICES = ["cpu", pytest.param("cuda:0", marks=pytest.mark.gpu)]
+F64 = torch.float64
+V = 83
+
+
+def base_cfg(**kw):
+    """Four stored layers (latent attention, delta, mamba2, latent attention
+    without a feed-forward), the middle two looped twice, three streams."""
+    args = dict(pattern="ldml", layers=4, loop=(1, 3, 2), streams=3, heads=3,
+                dim=12, rot_dim=8, vdim=20, kv_rank=24, q_rank=20,
+                delta_heads=4, delta_kv_heads=2, delta_dim=8, delta_vdim=12,
+                ssm_heads=6, ssm_vdim=4, ssm_state=8, ssm_groups=2,
+                norm_groups=3, conv=3, experts=5, top=2, expert_ff=24,
+                router_scale=1.5, embedding_scale=3.0, rot_base=300.0)
+    args.update(kw)
+    cfg = komizen_config(48, V, **args)
+    cfg["layers"] = copy.deepcopy(cfg["layers"])
+    if len(cfg["layers"]) == 4:
+        cfg["layers"][3]["mlp"] = None
+    return cfg
+
+
+def steady_cfg(dtype, **kw):
+    """The base stack; for bfloat16 runs a shallower one (every layer of these
+    tiny random models multiplies rounding noise by about 1.6) with one wide
+    norm group in the state-space layer."""
+    if dtype == "bfloat16":
+        kw = dict(dict(pattern="ldm", layers=3, loop=(1, 2, 2), norm_groups=1,
+                       ssm_vdim=8, ssm_groups=1), **kw)
+    return base_cfg(**kw)
+
+
+def tokens(n, seed, vocab=V):
+    return torch.randint(0, vocab, (n,),
+                         generator=torch.Generator().manual_seed(seed))
+
+
+def executor(cfg, sd, device, dtype="float32", slots=3, smax=160, **kw):
+    mc = ModelConfig.from_hf(cfg)
+    mc.compute_dtype = dtype
+    ex = RingExecutor(mc, 0, 1, torch.device(device), mb_size=slots,
+                      smax=smax, init_weights=False,
+                      use_graphs=kw.pop("use_graphs", False), **kw)
+    ex.model.load_state_dict(sd)
+    return ex
+
+
+def close(got, want, dtype="float32"):
+    got, want = got.detach().cpu().to(F64), want.to(F64)
+    scale = float(want.pow(2).mean().sqrt())
+    # float32 is the sharp comparison (the oracle run in float32 differs from
+    # its float64 self by up to 5e-4 of the scale on these stacks). In
+    # bfloat16 these tiny random stacks multiply rounding noise by about 1.6
+    # per layer and single positions stand out (the framework's own prompt
+    # and decode paths agree there to the last bit on the CPU), so the bound
+    # is on the root mean square, with a loose cap on any one entry.
+    if dtype == "float32":
+        cap, mean = 2e-3, 6e-4
+    else:
+        cap, mean = 1.0, 0.15
+    err = float((got - want).abs().max())
+    assert err <= cap * scale, f"max err {err:.3g} vs scale {scale:.3g}"
+    rms = float((got - want).pow(2).mean().sqrt())
+    assert rms <= mean * scale, f"rms err {rms:.3g} vs {scale:.3g}"
+
+
+def decode_step(ex, slot_tokens):
+    """One slot-batch decode step {slot: token}; other rows sit it out."""
+    tb = ex.tokbuf[0].cpu()
+    for s, t in slot_tokens.items():
+        tb[s] = int(t)
+    ex.tokbuf[0].copy_(tb)
+    idle = torch.ones(ex.mb_size, dtype=torch.bool)
+    idle[list(slot_tokens)] = False
+    idle = idle.to(ex.device)
+    ex.slot_step_compute(park=idle)
+    lg = ex.logits_buf[0].float().cpu().clone()
+    ex.kvs[0].pos.add_((~idle).to(torch.int32))
+    return lg
+
+
+def oracle(toks, cfg, sd, **kw):
+    return O.forward(cfg, sd, [int(t) for t in toks], F64, **kw)
+
+
+# ---------- configuration ----------
+
+def test_config_registry_and_loop_unrolling():
+    from dnet_amd.models import KomizenRingModel, get_ring_model
+    cfg = base_cfg()
+    mc = ModelConfig.from_hf(cfg)
+    assert mc.model_type == "komizen" and mc.num_layers == 6
+    assert mc.layer_weight_ids == [0, 1, 2, 1, 2, 3] and mc.hc_streams == 3
+    assert mc.stored_layers([3, 4]) == [1, 2]
+    assert get_ring_model("komizen") is KomizenRingModel
+    plain = base_cfg(loop=None, streams=0)
+    mp = ModelConfig.from_hf(plain)
+    assert mp.layer_weight_ids == [0, 1, 2, 3] and mp.hc_streams == 0
+    for path, value in ((("layers", 0, "type"), "conv"),
+                        (("layers", 1, "mlp", "kind"), "dense"),
+                        (("layers", 1, "mixer", "kv_heads"), 3),
+                        (("layers", 0, "mixer", "rot", "dims"), 6),
+                        (("loop", "stop"), 9)):
+        bad = base_cfg()
+        node = bad
+        for k in path[:-1]:
+            node = node[k]
+        node[path[-1]] = value
+        with pytest.raises(ValueError):
+            ModelConfig.from_hf(bad)
+    # runs of a looped layer share one weight object and own separate state
+    sd = O.make_checkpoint(cfg, 1)
+    ex = executor(cfg, sd, "cpu")
+    m = ex.model
+    assert m.layers[1] is m.layers[3] and m.layers[2] is m.layers[4]
+    st = ex.kvs[0].state
+    assert st[1]["S"].data_ptr() != st[3]["S"].data_ptr()
+    assert ex.kvs[0].k[0].shape[-1] == 24 + 8 and ex.kvs[0].v[0] is None
+    assert ex.hbuf[0].shape[1] == 3 * 48
+
+
+# ---------- mechanisms alone ----------
+
+def _one_layer(kind, **kw):
+    cfg = base_cfg(pattern=kind, layers=1, loop=None, **kw)
+    return cfg
+
+
+def _mixer_alone(device, cfg, sd, u, T0, portion=None):
+    """Run the layer's mixer on given inputs u [T, W] through the cache: the
+    first T0 rows as one prompt portion (or portions), then row by row."""
+    ex = executor(cfg, sd, device)
+    m, kv = ex.model, ex.kvs[0]
+    lw, spec = m.layers[0], m.cfg.layer_specs[0]
+    fn = {"latent_attention": m._latent_attention, "delta": m._delta,
+          "mamba2": m._ssd}[spec["type"]]
+    T = u.shape[0]
+    slot = torch.tensor([2], dtype=torch.int32, device=device)
+    steps, p = [], 0
+    while p < T0:
+        n = min(portion or T0, T0 - p)
+        steps.append((p, n))
+        p += n
+    steps += [(t, 1) for t in range(T0, T)]
+    outs = []
+    for p0, n in steps:
+        pos = torch.tensor([p0], dtype=torch.int32, device=device)
+        ln = torch.tensor([n], dtype=torch.int32, device=device)
+        x = u[p0:p0 + n].to(torch.float32).to(device).contiguous()
+        outs.append(fn(x, lw, spec["mixer"], kv, 0, pos, n, ln, slot)
+                    .float().cpu())
+    return torch.cat(outs)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("kind,kw", [
+    ("d", {}), ("d", dict(delta_heads=3, delta_kv_heads=3, delta_dim=5,
+                          delta_vdim=7, conv=2)),
+    ("d", dict(delta_heads=2, delta_kv_heads=1, delta_dim=32, delta_vdim=16,
+               conv=5)),
+    ("m", {}), ("m", dict(ssm_heads=2, ssm_vdim=9, ssm_state=5, ssm_groups=1,
+                          norm_groups=1, conv=4)),
+    ("l", {}), ("l", dict(heads=1, dim=4, rot_dim=2, vdim=3, kv_rank=7,
+                          q_rank=5)),
+    ("l", dict(heads=4, dim=16, rot_dim=16, vdim=8, kv_rank=40, q_rank=12)),
+])
+def test_each_mixer_alone(device, kind, kw):
+    """A mixer on its own inputs: prompt portion, then token by token through
+    the cache / state, equals the oracle's whole-sequence result."""
+    cfg = _one_layer(kind, **kw)
+    sd = O.make_checkpoint(cfg, 3)
+    T = 41
+    u = torch.randn(T, 48, generator=torch.Generator().manual_seed(9))
+    spec = cfg["layers"][0]
+    want = O.MIXERS[spec["type"]](u.to(F64), O.sub(sd, "l0.mix.", F64),
+                                  spec["mixer"], cfg["norm"]["eps"])
+    for T0, portion in ((29, None), (30, 7), (2, 2)):
+        got = _mixer_alone(device, cfg, sd, u, T0, portion)
+        close(got, want)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_far_key_and_rotation_at_long_distance(device):
+    """One early key is made to dominate (its unnormed rotated part is
+    scaled up), so every later query, hundreds of positions on, must find it
+    with the right relative angle; prompt rows and decoded rows."""
+    cfg = _one_layer("l", heads=2, dim=8, rot_dim=8, vdim=8, kv_rank=16,
+                     q_rank=12, rot_base=50.0)
+    sd = O.make_checkpoint(cfg, 4)
+    T = 300
+    u = torch.randn(T, 48, generator=torch.Generator().manual_seed(2))
+    u[3] *= 25.0
+    spec = cfg["layers"][0]
+    want = O.MIXERS["latent_attention"](
+        u.to(F64), O.sub(sd, "l0.mix.", F64), spec["mixer"], 1e-6)
+    ex_smax = 320
+    mc = ModelConfig.from_hf(cfg)
+    mc.compute_dtype = "float32"
+    got = None
+    for T0, portion in ((290, None), (288, 64)):
+        ex = RingExecutor(mc, 0, 1, torch.device(device), mb_size=3,
+                          smax=ex_smax, init_weights=False, use_graphs=False)
+        ex.model.load_state_dict(sd)
+        m, kv = ex.model, ex.kvs[0]
+        slot = torch.tensor([1], dtype=torch.int32, device=device)
+        outs, p = [], 0
+        steps = []
+        while p < T0:
+            n = min(portion or T0, T0 - p)
+            steps.append((p, n))
+            p += n
+        steps += [(t, 1) for t in range(T0, T)]
+        for p0, n in steps:
+            pos = torch.tensor([p0], dtype=torch.int32, device=device)
+            ln = torch.tensor([n], dtype=torch.int32, device=device)
+            outs.append(m._latent_attention(
+                u[p0:p0 + n].to(device).contiguous(), m.layers[0],
+                spec["mixer"], kv, 0, pos, n, ln, slot).float().cpu())
+        got = torch.cat(outs)
+        close(got, want)
+    # the far key really carries weight: without it the result moves
+    u2 = u.clone()
+    u2[3] /= 25.0
+    other = O.MIXERS["latent_attention"](
+        u2.to(F64), O.sub(sd, "l0.mix.", F64), spec["mixer"], 1e-6)
+    assert float((other[200:] - want[200:]).abs().max()) > 0.05
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("rows", [1, 3, 9, 70])
+@pytest.mark.parametrize("top,experts", [(2, 5), (1, 4), (3, 3)])
+def test_expert_routing(device, rows, top, experts):
+    """Softmax over all experts, the largest kept, weights not renormalized,
+    times the constant: every code path by row count (grouped kernels, batched
+    products, per-expert gathers)."""
+    cfg = _one_layer("d", experts=experts, top=top, router_scale=0.7)
+    sd = O.make_checkpoint(cfg, 5)
+    ex = executor(cfg, sd, device)
+    m = ex.model
+    u = torch.randn(rows, 48, generator=torch.Generator().manual_seed(rows))
+    got = m._moe(u.to(device), m.layers[0], cfg["layers"][0]["mlp"])
+    want = O.moe_ff(u.to(F64), O.sub(sd, "l0.mlp.", F64),
+                    cfg["layers"][0]["mlp"])
+    close(got, want)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("S", [1, 2, 4])
+def test_stream_read_write(device, S):
+    import dnet_amd.ops as ops
+    g = torch.Generator().manual_seed(S)
+    M, W = 6, 20
+    xs = [torch.randn(M, W, generator=g, dtype=F64) for _ in range(S)]
+    y = torch.randn(M, W, generator=g, dtype=F64)
+    a, b = torch.randn(S, generator=g), torch.randn(S, generator=g)
+    mix = torch.randn(S, S, generator=g)
+    wn = torch.randn(W, generator=g)
+    packed = torch.cat(xs, dim=1).float().to(device).contiguous()
+    nxt = ops.hc_write(packed, y.float().to(device), mix.to(device),
+                       b.to(device), a.to(device), (1 + wn).to(device), 1e-6,
+                       torch.float32)
+    new = [sum(mix[s, t].double() * xs[s] for s in range(S))
+           + b[t].double() * y for t in range(S)]
+    close(packed.cpu(), torch.cat(new, dim=1))
+    u = sum(a[t].double() * new[t] for t in range(S))
+    close(nxt.cpu(), O.norm_centered(u, wn.double(), 1e-6))
+
+
+# ---------- whole model ----------
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prompt_logits_first_tokens_and_layers(device, dtype):
+    cfg = steady_cfg(dtype)
+    sd = O.make_checkpoint(cfg, 6, ff_gain=1.0 if dtype == "float32" else 0.1)
+    a = tokens(37, 1)
+    layers = []
+    want = oracle(a, cfg, sd, layers_out=layers)
+    ex = executor(cfg, sd, device, dtype)
+    got = ex.prefill_slots([1], [a], want=[list(range(37))])[0]
+    close(got, want, dtype)
+    if dtype == "float32":
+        # the sum of the streams after every layer run
+        m, kv = ex.model, ex.kvs[0]
+        h = m.embed_tokens(a.view(1, -1).to(device)).clone()
+        ln = torch.tensor([37], dtype=torch.int32, device=device)
+        slot = torch.tensor([2], dtype=torch.int32, device=device)
+        for run in range(6):
+            m.prefill_window(h, [run], kv, 0, lens=ln, slots=slot)
+            close(h.view(37, 3, 48).sum(1), layers[run])
+    # single-token prompts and the very first positions
+    one = ex.prefill_slots([0], [a[:1]])[0]
+    close(one, want[:1], dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_prefill_vs_token_by_token_and_long_decode(device):
+    cfg = base_cfg()
+    sd = O.make_checkpoint(cfg, 7)
+    a = tokens(150, 2)
+    want = oracle(a, cfg, sd)
+    ex = executor(cfg, sd, device)
+    got = [ex.prefill_slots([2], [a[:1]])[0]]
+    for t in range(1, 150):                 # decode from the second token on
+        got.append(decode_step(ex, {2: a[t]})[2:3])
+    close(torch.cat(got), want)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("chunk", [2, 3, 16, 33])
+def test_portions(device, chunk):
+    """A prompt cut into portions (executor chunking and continued requests)
+    gives the logits of the whole prompt."""
+    cfg = base_cfg()
+    sd = O.make_checkpoint(cfg, 8)
+    a = tokens(45, 3)
+    want = oracle(a, cfg, sd)
+    ex = executor(cfg, sd, device)
+    got = ex.prefill_slots([1], [a], want=[list(range(45))], chunk=chunk)[0]
+    close(got, want)
+    # the same through continued calls of unequal size
+    rows, p = [], 0
+    for n in (chunk, 2, 45):
+        n = min(n, 45 - p)
+        if n <= 0:
+            break
+        rows.append(ex.prefill_slots([0], [a[p:p + n]],
+                                     want=[list(range(n))], start=[p])[0])
+        p += n
+    close(torch.cat(rows), want[:p])
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_unequal_batch_equals_each_alone(device, dtype):
+    cfg = steady_cfg(dtype)
+    sd = O.make_checkpoint(cfg, 9, ff_gain=1.0 if dtype == "float32" else 0.1)
+    a, b, c = tokens(40, 4), tokens(5, 5), tokens(1, 6)
+    if dtype == "float32":
+        wa, wb, wc = (oracle(t, cfg, sd) for t in (a, b, c))
+    else:
+        # each request alone through the framework, whole and in one step
+        wa, wb, wc = (executor(cfg, sd, device, dtype).prefill_slots(
+            [0], [t], want=[list(range(len(t)))])[0].float().cpu()
+            for t in (a, b, c))
+    ex = executor(cfg, sd, device, dtype, slots=4)
+    got = ex.prefill_slots([3, 1, 0], [a[:30], b[:3], c],
+                           want=[[0, 29], [2], [0]])
+    close(got[0], wa[[0, 29]], dtype)
+    close(got[1], wb[2:3], dtype)
+    close(got[2], wc, dtype)
+    for i in range(2):                      # decoded together
+        lg = decode_step(ex, {3: a[30 + i], 1: b[3 + i]})
+        close(lg[3:4], wa[30 + i].view(1, -1), dtype)
+        close(lg[1:2], wb[3 + i].view(1, -1), dtype)
+    for i in range(32, 40):                 # the shorter request has ended
+        lg = decode_step(ex, {3: a[i]})
+        close(lg[3:4], wa[i].view(1, -1), dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_slot_freed_and_used_again(device):
+    """A slot that held a long request is taken by a new one without any
+    reset: cache rows and recurrent states of the old request do not leak."""
+    cfg = base_cfg()
+    sd = O.make_checkpoint(cfg, 10)
+    a, b = tokens(60, 7), tokens(20, 8)
+    ex = executor(cfg, sd, device, slots=2)
+    ex.prefill_slots([1], [a[:50]])
+    for t in range(50, 60):
+        decode_step(ex, {1: a[t]})
+    wb = oracle(b, cfg, sd)
+    ex.kvs[0].pos[1] = 0
+    got = ex.prefill_slots([1], [b[:12]], want=[[0, 5, 11]])[0]
+    close(got, wb[[0, 5, 11]])
+    for t in range(12, 20):
+        close(decode_step(ex, {1: b[t]})[1:2], wb[t].view(1, -1))
+
+
+OTHER = [
+    # one stream with its own weights; loop of three passes over one layer
+    dict(streams=1, pattern="md", layers=2, loop=(0, 1, 3), ssm_groups=1,
+         norm_groups=1, conv=2, top=1, experts=3),
+    # no streams (plain residual), no loop, every router choice taken
+    dict(streams=0, loop=None, pattern="ldm", layers=3, top=4, experts=4,
+         heads=2, dim=6, rot_dim=4, vdim=5, kv_rank=10, q_rank=9),
+    # key heads equal to value heads, rotated part wider than the plain one
+    dict(streams=4, pattern="dl", layers=2, loop=(1, 2, 2), delta_heads=2,
+         delta_kv_heads=2, delta_dim=6, delta_vdim=10, heads=5, dim=4,
+         rot_dim=12, vdim=6, kv_rank=9, q_rank=7, conv=5),
+]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("kw", OTHER)
+def test_other_sizes(device, kw):
+    cfg = base_cfg(**kw)
+    sd = O.make_checkpoint(cfg, 11)
+    a, b = tokens(33, 9), tokens(7, 10)
+    wa, wb = oracle(a, cfg, sd), oracle(b, cfg, sd)
+    ex = executor(cfg, sd, device, slots=2)
+    got = ex.prefill_slots([0, 1], [a[:25], b[:4]],
+                           want=[list(range(25)), [3]], chunk=9)
+    close(got[0], wa[:25])
+    close(got[1], wb[3:4])
+    for i in range(3):
+        lg = decode_step(ex, {0: a[25 + i], 1: b[4 + i]})
+        close(lg[0:1], wa[25 + i].view(1, -1))
+        close(lg[1:2], wb[4 + i].view(1, -1))
+
+
+@pytest.mark.gpu
+def test_decode_graph_replays_match_eager():
+    """Captured decode steps, replayed with eager prefills and host syncs in
+    between, equal the eager steps every time (warm-up runs of the capture
+    must not advance any slot's state)."""
+    cfg = steady_cfg("bfloat16")
+    sd = O.make_checkpoint(cfg, 12, ff_gain=0.1)
+    a, b = tokens(40, 31), tokens(30, 32)
+    runs = []
+    for graphs in (False, True):
+        ex = executor(cfg, sd, "cuda:0", "bfloat16", use_graphs=graphs)
+        out = [ex.prefill_slots([1], [a[:30]], want=[[0, 29]])[0].float().cpu()]
+        for t in range(30, 35):
+            out.append(decode_step(ex, {1: a[t]})[1:2])
+        out.append(ex.prefill_slots([2], [b[:25]],
+                                    want=[[3, 24]])[0].float().cpu())
+        for t in range(5):
+            lg = decode_step(ex, {1: a[35 + t], 2: b[25 + t]})
+            out.append(lg[1:3])
+            torch.cuda.synchronize()
+        runs.append(torch.cat(out))
+    torch.testing.assert_close(runs[1], runs[0], atol=2e-2, rtol=2e-2)
+
+
+# ---------- generation through the scheduler, trace replay ----------
+
+def write_checkpoint(path: Path, cfg, sd):
+    from safetensors.torch import save_file
+    path.mkdir(parents=True, exist_ok=True)
+    (path / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.contiguous() for k, v in sd.items()},
+              str(path / "model.safetensors"))
+
+
+def oracle_greedy(prompt, n, cfg, sd):
+    seq = list(prompt)
+    for _ in range(n):
+        seq.append(int(oracle(seq, cfg, sd)[-1].argmax()))
+    return seq[len(prompt):]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_greedy_generation_through_slot_scheduler(tmp_path, device,
+                                                  monkeypatch):
+    """Requests queued at the shard runtime are admitted into slots (more
+    requests than slots), prefilled, decoded as one batch with idle rows in
+    it and sampled greedily; every token equals the oracle's argmax."""
+    if device == "cpu":
+        monkeypatch.setattr(torch.cuda, "is_available", lambda: False)
+    from dnet_amd.core.types import ShardLoadModelRequest
+    from dnet_amd.shard.runtime import ShardRuntime
+    cfg = base_cfg()
+    cfg["vocab"] = 59
+    sd = O.make_checkpoint(cfg, 15)
+    write_checkpoint(tmp_path / "m", cfg, sd)
+    emitted: dict = {}
+
+    class Cap:
+        def send(self, frame):
+            emitted.setdefault(frame["nonce"], []).append(
+                (frame["token_id"], frame["finished"]))
+
+        def close(self):
+            pass
+
+    rt = ShardRuntime("probe")
+    monkeypatch.setattr(rt.settings.storage, "repack_on_load", False)
+    rt._load(ShardLoadModelRequest(
+        model_path=str(tmp_path / "m"), total_layers=6,
+        layers=list(range(6)), max_batch=2, max_seq=96, dtype="float32"))
+    assert (rt.executor.device.type == "cuda") == device.startswith("cuda")
+    rt._callback = Cap()
+    prompts = {"a": tokens(9, 1, 59), "b": tokens(2, 2, 59),
+               "c": tokens(23, 3, 59)}
+    n_new = {"a": 6, "b": 9, "c": 4}
+    for name in ("a", "b", "c"):            # c waits for a slot to free up
+        rt.infer_q.put({"nonce": name, "prompt_len": len(prompts[name]),
+                        "tokens": prompts[name].to(torch.int32).numpy()
+                        .tobytes(), "max_tokens": n_new[name],
+                        "stop_ids": [], "params": {}})
+    for _ in range(60):
+        rt._slots_tick()
+        if all(emitted.get(k) and emitted[k][-1][1] for k in prompts):
+            break
+    for name, p in prompts.items():
+        got = [t for t, _ in emitted[name]]
+        assert got == oracle_greedy(p.tolist(), n_new[name], cfg, sd), name
+    rt._unload()
+
+
+@pytest.mark.gpu
+def test_trace_replay_cli_gpu(tmp_path):
+    test_trace_replay_cli(tmp_path, "bfloat16")
+    test_trace_replay_cli(tmp_path / "f", "float32")
+
+
+def test_trace_replay_cli(tmp_path, dtype="float32"):
+    """bin/trace_run on a tiny checkpoint: a prompt batch of unequal
+    requests (more than the initial slot count), decode steps together, a
+    request that sits steps out, requests that end early, a slot used
+    again by a new request."""
+    cfg = steady_cfg(dtype)
+    cfg["vocab"] = 53
+    sd = O.make_checkpoint(cfg, 16,
+                           ff_gain=1.0 if dtype == "float32" else 0.1)
+    write_checkpoint(tmp_path / "m", cfg, sd)
+    a, b = tokens(14, 1, 53).tolist(), tokens(4, 2, 53).tolist()
+    c, d = tokens(12, 3, 53).tolist(), tokens(6, 4, 53).tolist()
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:11], "want": [0, 10]},
+                                {"id": "b", "tokens": b[:2], "want": []},
+                                {"id": "c", "tokens": c[:10], "want": [9]}],
+         "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[11:12], "want": [0]},
+                                {"id": "b", "tokens": b[2:3], "want": [0]}],
+         "end": []},
+        {"step": 2, "entries": [{"id": "a", "tokens": a[12:13], "want": []},
+                                {"id": "b", "tokens": b[3:4], "want": [0]}],
+         "end": ["b"]},
+        {"step": 3, "entries": [{"id": "a", "tokens": a[13:14], "want": [0]}],
+         "end": ["a"]},
+        {"step": 4, "entries": [{"id": "c", "tokens": c[10:11], "want": [0]}],
+         "end": []},
+        {"step": 5, "entries": [{"id": "d", "tokens": d[:5], "want": [4]}],
+         "end": []},
+        {"step": 6, "entries": [{"id": "c", "tokens": c[11:12], "want": [0]},
+                                {"id": "d", "tokens": d[5:6], "want": [0]}],
+         "end": ["c", "d"]},
+    ]
+    root = Path(__file__).resolve().parents[1]
+    r = subprocess.run(
+        [sys.executable, str(root / "bin" / "trace_run"), "--model",
+         str(tmp_path / "m"), "--dtype", dtype, "--out",
+         str(tmp_path / "out"), "--max-tokens", "48", "--max-batch", "2"],
+        input="\n".join(json.dumps(s) for s in steps) + "\n", text=True,
+        capture_output=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == [
+        f"done {i}" for i in range(7)]
+    w = {n: oracle(t, cfg, sd) for n, t in
+         (("a", a), ("b", b), ("c", c), ("d", d))}
+    import numpy as np
+
+    def rd(i):
+        return torch.from_numpy(np.fromfile(tmp_path / "out" / f"{i}.f32",
+                                            dtype="<f4").reshape(-1, 53))
+    close(rd(0), torch.cat([w["a"][[0, 10]], w["c"][9:10]]), dtype)
+    close(rd(1), torch.stack([w["a"][11], w["b"][2]]), dtype)
+    close(rd(2), w["b"][3:4], dtype)
+    close(rd(3), w["a"][13:14], dtype)
+    close(rd(4), w["c"][10:11], dtype)
+    close(rd(5), w["d"][4:5], dtype)
+    close(rd(6), torch.stack([w["c"][11], w["d"][5]]), dtype)
+
+
+# ---------- pipeline stages (gloo, two processes) ----------
+
+def _ring_run(rank, world):
+    cfg = base_cfg()
+    mc = ModelConfig.from_hf(cfg)
+    mc.compute_dtype = "float32"
+    ex = RingExecutor(mc, rank, world, "cpu", mb_count=1, mb_size=2, smax=64,
+                      seed=7, use_graphs=False)
+    g = torch.Generator().manual_seed(21)
+    first = ex.prefill(torch.randint(0, V, (1, 2, 13), generator=g), chunk=5)
+    steps = []
+    ex.decode_stream(6, on_token=lambda s, t, last: steps.append(t.clone()))
+    if rank:
+        return None
+    return torch.cat([first.view(2, 1)] + [t.view(2, 1) for t in steps], -1)
+
+
+def _ring_rank_main(rank, world, port, q):
+    import os
+    os.environ.update(RANK=str(rank), WORLD_SIZE=str(world),
+                      MASTER_ADDR="127.0.0.1", MASTER_PORT=str(port),
+                      LOCAL_RANK=str(rank))
+    import torch.distributed as dist
+    dist.init_process_group("gloo", rank=rank, world_size=world)
+    out = _ring_run(rank, world)
+    if rank == 0:
+        q.put(out)
+    dist.destroy_process_group()
+
+
+@pytest.mark.timeout(360)
+def test_two_stage_ring_matches_single():
+    """Layer runs split over two pipeline stages (the looped span is cut in
+    the middle): all residual streams ride the ring hops and the generated
+    tokens equal the single-stage run."""
+    import multiprocessing as mp
+    import socket
+    single = _ring_run(0, 1)
+    s = socket.socket()
+    s.bind(("127.0.0.1", 0))
+    port = s.getsockname()[1]
+    s.close()
+    ctx = mp.get_context("spawn")
+    q = ctx.Queue()
+    procs = [ctx.Process(target=_ring_rank_main, args=(r, 2, port, q))
+             for r in range(2)]
+    for p in procs:
+        p.start()
+    out = q.get(timeout=200)
+    for p in procs:
+        p.join(timeout=60)
+        assert p.exitcode == 0
+    assert single.shape[0] == 2 and single.shape[1] >= 6
+    assert torch.equal(out, single)
+
+
+def test_synthetic_preset_runs():
+    """The preset builds with seeded random weights and generates the same
+    tokens whatever the slot a prompt sits in."""
+    from dnet_amd.models import PRESETS
+    mc = ModelConfig.from_hf(dict(PRESETS["komizen-tiny"]))
+    ex = RingExecutor(mc, 0, 1, "cpu", mb_size=2, smax=96, seed=3,
+                      use_graphs=False)
+    toks = torch.randint(0, 256, (1, 2, 30),
+                         generator=torch.Generator().manual_seed(1))
+    toks[0, 1] = toks[0, 0]
+    first = ex.prefill(toks)
+    gen = ex.decode_rounds(6)
+    assert torch.equal(first[0, 0], first[0, 1])
+    assert torch.equal(gen[0, 0], gen[0, 1])
+    with pytest.raises(NotImplementedError):
+        RingExecutor(mc, 0, 1, "cpu", mb_size=1, smax=32, residency=2,
+                     use_graphs=False)

@@ -155,7 +155,8 @@ def _executors(dtype, mb=3, smax=192):
                         experts=5, top=2, expert_ff=48, router_scale=1.5,
                         embedding_scale=3.0)
     from komizen_oracle import make_checkpoint
-    sd = make_checkpoint(hf, seed=11)
+    sd = make_checkpoint(hf, seed=11,
+                         ff_gain=1.0 if dtype == "float32" else 0.1)
     out = []
     for dev, graphs in (("cpu", False), (DEV, True)):
         cfg = ModelConfig.from_hf(hf)
