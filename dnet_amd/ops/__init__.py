@@ -540,9 +540,24 @@ def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
             if window:
                 span = min(span, window + 64
                            + (pool_k.shape[2] if pool else 0))
-            splits = _attn_mod_splits(q.shape[0] * Hkv * -(-(Hq // Hkv) // 16),
-                                      span)
-            if splits > 1:
+            G = Hq // Hkv
+            if (q.dtype == torch.bfloat16 and G >= 16 and not pool
+                    and D % 8 == 0 and Dv % 8 == 0):
+                # grouped heads on the matrix cores (the extension picks the
+                # kernel by the same rule): 64 heads per workgroup, splits of
+                # at least 128 keys of capacity (measured: more splits cost
+                # more in the merge than they gain), partials at every split
+                # count
+                splits = 1
+                blocks = q.shape[0] * Hkv * -(-G // 64)
+                while blocks * splits < 1024 and splits * 256 <= span:
+                    splits *= 2
+                partials = torch.empty(q.shape[0] * Hq * splits * (Dv + 2),
+                                       dtype=torch.float32, device=q.device)
+            else:
+                splits = _attn_mod_splits(q.shape[0] * Hkv * -(-G // 16),
+                                          span)
+            if splits > 1 and partials is None:
                 partials = torch.empty(q.shape[0] * Hq * splits * (Dv + 2),
                                        dtype=torch.float32, device=q.device)
         _native().attn_mod(q, kcache, vcache, pos, lens, slots, out, T,

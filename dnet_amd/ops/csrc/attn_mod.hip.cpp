@@ -17,7 +17,7 @@
 // (block means written by kv_pool_update) for every c < (i - window + 1) /
 // pool, in the same softmax and without a distance penalty.
 //
-// Two kernels:
+// Three kernels:
 //  * attn_mod_rows<T>: flash-decode layout. One workgroup per (q tile, kv
 //    head, batch row): K/V chunks of 64 positions are staged through LDS once
 //    and shared by up to 16 query rows (tokens x grouped heads); score phase =
@@ -27,6 +27,9 @@
 //  * attn_mod_mfma<DC,NV>: bf16 prefill on v_mfma_f32_16x16x32_bf16 — QK^T
 //    and PV on the matrix cores, modifiers + online softmax in the fp32 C
 //    fragments. Head sizes are zero-padded in LDS to DC*32 / NV*16.
+//  * attn_mod_mfma_heads<DC,NV>: bf16 decode with >= 16 query heads per kv
+//    head (latent attention's one shared row): the grouped heads are the rows
+//    of the MFMA tile, split over the keys.
 #include "common.h"
 
 namespace dnet {
@@ -82,6 +85,8 @@ __device__ __forceinline__ float dot_lds(const short* a, const short* b, int n) 
 
 constexpr int kChunkR = 64;   // keys per staged chunk (one per lane)
 constexpr int kRowsMax = 16;  // query rows per workgroup (4 per wave)
+constexpr int kHeadsMfmaMinGroup = 16;  // decode: heads per kv head from which
+                                        // the matrix-core heads kernel runs
 
 __host__ __device__ inline int pitch_of(int n, int elem) {
   // fp32: odd dword pitch; bf16: 8 B aligned rows with a 2-dword skew
@@ -591,6 +596,210 @@ __global__ __launch_bounds__(256) void attn_mod_mfma(
   }
 }
 
+// ---- bf16 decode of grouped heads on the matrix cores ----------------------
+// One token per batch row (T = 1) and many query heads per kv head (latent
+// attention: every head reads the one shared row): the G grouped heads are
+// the 16 rows of a wave's MFMA tile (4 waves = 64 heads per block), so a
+// staged 32-key K/V tile is used by all of them. grid (splits, Hkv * head
+// tiles, B); key tiles are dealt round robin to the splits and unnormalized
+// (acc, m, l) go to `partial` [B, Hq, splits, DV+2] for attn_mod_combine
+// (which also adds the sink). No pooled entries.
+template <int DC, int NV>
+__global__ __launch_bounds__(256) void attn_mod_mfma_heads(
+    const short* __restrict__ q, const short* __restrict__ kc,
+    const short* __restrict__ vc, float* __restrict__ partial,
+    const int splits, const ModParams P) {
+  constexpr int ST = 32;
+  constexpr int DP = DC * 32, DVP = NV * 16;
+  constexpr int KP = DP + 8, SP = ST + 8;
+  __shared__ short k_lds[ST * KP];
+  __shared__ short vt_lds[DVP * SP];
+  __shared__ short p_lds[4][16 * SP];
+
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int split = blockIdx.x, b = blockIdx.z;
+  const int G = P.Hq / P.Hkv;
+  const int GT = (G + 63) / 64;
+  const int hk = blockIdx.y / GT;
+  const int gw = (blockIdx.y % GT) * 64 + wave * 16;   // wave's first head
+  const int D = P.D, DV = P.DV, VS = P.VS;
+  if (P.lens && P.lens[b] <= 0) return;                // idle row
+  const int slot = P.slots ? P.slots[b] : b;
+  if (slot < 0 || slot >= P.Bc) return;
+  const int i = P.pos[b];                              // the query's position
+  const int row = lane & 15, hi = lane >> 4;
+  const int hrow = hk * G + min(gw + row, G - 1);
+  const short* qp = q + ((int64_t)b * P.Hq + hrow) * D;
+  const short* kp = kc + ((int64_t)slot * P.Hkv + hk) * P.Smax * D;
+  const short* vp = vc + ((int64_t)slot * P.Hkv + hk) * P.Smax * VS;
+
+  bf16x8 qf[DC];
+#pragma unroll
+  for (int c = 0; c < DC; ++c) {
+    const int e0 = c * 32 + hi * 8;
+    short8 z;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) z.x[j] = 0;
+    if (e0 < D) z = *reinterpret_cast<const short8*>(&qp[e0]);
+    qf[c] = *reinterpret_cast<const bf16x8*>(&z);
+  }
+  f32x4 acc[NV];
+#pragma unroll
+  for (int nn = 0; nn < NV; ++nn) acc[nn] = {0.f, 0.f, 0.f, 0.f};
+  float m_run[4], l_run[4], sc_t[4], r1[4], r2[4];
+  bool alive[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int g = gw + hi * 4 + r;
+    alive[r] = g < G;
+    const int h = hk * G + min(g, G - 1);
+    sc_t[r] = P.scale * (P.temp ? P.temp[h] : 1.f);
+    r1[r] = P.r1 ? P.r1[h] : 0.f;
+    r2[r] = P.r1 ? P.r2[h] : 0.f;
+    m_run[r] = -1e30f;
+    l_run[r] = 0.f;
+  }
+  const float cap = P.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
+
+  const int s_end = min(P.Smax, i + 1);
+  const int s_begin = P.window > 0 ? (max(0, i - P.window + 1) & ~(ST - 1)) : 0;
+  const int tiles = s_end > s_begin ? (s_end - s_begin + ST - 1) / ST : 0;
+
+  // the next tile's key rows travel from memory into registers while the
+  // current tile is worked on
+  constexpr int KV = ST * (DP / 8) / 256;       // 16 B pieces per thread
+  short8 kreg[KV];
+  auto load_tile = [&](const int s0) {
+#pragma unroll
+    for (int v = 0; v < KV; ++v) {
+      const int idx = threadIdx.x + v * 256;
+      const int sr = idx / (DP / 8), dc = (idx % (DP / 8)) * 8;
+      const int sg = min(s0 + sr, P.Smax - 1);
+      short8 z;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) z.x[j] = 0;
+      if (dc < D) z = *reinterpret_cast<const short8*>(&kp[(int64_t)sg * D + dc]);
+      kreg[v] = z;
+    }
+  };
+  if (split < tiles) load_tile(s_begin + split * ST);
+
+  for (int tile = split; tile < tiles; tile += splits) {
+    const int s0 = s_begin + tile * ST;
+    __syncthreads();
+#pragma unroll
+    for (int v = 0; v < KV; ++v) {
+      const int idx = threadIdx.x + v * 256;
+      const int sr = idx / (DP / 8), dc = (idx % (DP / 8)) * 8;
+      *reinterpret_cast<short8*>(&k_lds[sr * KP + dc]) = kreg[v];
+    }
+    if (tile + splits < tiles) load_tile(s0 + splits * ST);
+    if (P.vshare) {
+      // the staged key rows are the values: transpose them inside LDS, the
+      // 32 keys of a value dimension across neighbouring lanes (consecutive
+      // writes, key rows 4 banks apart for the reads)
+      __syncthreads();
+      for (int idx = threadIdx.x; idx < ST * (DVP / 2); idx += 256) {
+        const int sr = idx % ST, dc = (idx / ST) * 2;
+        unsigned pr = 0;
+        if (dc < DV)              // DV is even (multiple of 8)
+          pr = *reinterpret_cast<const unsigned*>(&k_lds[sr * KP + dc]);
+        vt_lds[dc * SP + sr] = (short)(pr & 0xffffu);
+        vt_lds[(dc + 1) * SP + sr] = (short)(pr >> 16);
+      }
+    } else {
+      for (int idx = threadIdx.x; idx < ST * (DVP / 2); idx += 256) {
+        const int sr = idx / (DVP / 2), dc = (idx % (DVP / 2)) * 2;
+        const int sg = min(s0 + sr, P.Smax - 1);
+        short v0 = 0, v1 = 0;
+        if (dc < DV) {            // DV is even (multiple of 8)
+          v0 = vp[(int64_t)sg * VS + dc];
+          v1 = vp[(int64_t)sg * VS + dc + 1];
+        }
+        vt_lds[dc * SP + sr] = v0;
+        vt_lds[(dc + 1) * SP + sr] = v1;
+      }
+    }
+    __syncthreads();
+
+    float p_val[2][4], m_new[4];
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      f32x4 sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < DC; ++c) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(
+            &k_lds[(sub * 16 + row) * KP + c * 32 + hi * 8]);
+        sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[c], kf, sc, 0, 0, 0);
+      }
+      const int j = s0 + sub * 16 + row;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float val = sc[r] * sc_t[r];
+        if (cap > 0.f) val = cap * fast_tanh(val * inv_cap);
+        if (P.r1) val -= r1[r] * __logf(1.f + r2[r] * (float)max(i - j, 0));
+        bool dead = (j > i) || (j >= P.Smax) || !alive[r];
+        if (P.window > 0) dead |= (j <= i - P.window);
+        p_val[sub][r] = dead ? -INFINITY : val;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float mx = fmaxf(p_val[0][r], p_val[1][r]);
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1)
+        mx = fmaxf(mx, __shfl_xor(mx, off, 16));
+      m_new[r] = fmaxf(m_run[r], mx);
+      const float corr = __expf(m_run[r] - m_new[r]);
+      float ls = 0.f;
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub) {
+        p_val[sub][r] = __expf(p_val[sub][r] - m_new[r]);
+        ls += p_val[sub][r];
+      }
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1) ls += __shfl_xor(ls, off, 16);
+      l_run[r] = l_run[r] * corr + ls;
+      m_run[r] = m_new[r];
+#pragma unroll
+      for (int nn = 0; nn < NV; ++nn) acc[nn][r] *= corr;
+    }
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        p_lds[wave][(hi * 4 + r) * SP + sub * 16 + row] =
+            f2bits(p_val[sub][r]);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // wave-local slab
+    const bf16x8 pf =
+        *reinterpret_cast<const bf16x8*>(&p_lds[wave][row * SP + hi * 8]);
+#pragma unroll
+    for (int nn = 0; nn < NV; ++nn) {
+      const bf16x8 vf = *reinterpret_cast<const bf16x8*>(
+          &vt_lds[(nn * 16 + row) * SP + hi * 8]);
+      acc[nn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, acc[nn], 0,
+                                                        0, 0);
+    }
+  }
+
+  // a split without tiles still reports its neutral (0, -1e30, 0)
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    if (!alive[r]) continue;
+    const int h = hk * G + gw + hi * 4 + r;
+    float* pp = partial + (((int64_t)b * P.Hq + h) * splits + split) * (DV + 2);
+#pragma unroll
+    for (int nn = 0; nn < NV; ++nn) {
+      const int dv = nn * 16 + row;
+      if (dv < DV) pp[dv] = acc[nn][r];
+    }
+    if (row == 0) {
+      pp[DV] = m_run[r];
+      pp[DV + 1] = l_run[r];
+    }
+  }
+}
+
 }  // namespace
 
 static const float* opt_f32(const c10::optional<torch::Tensor>& t, int64_t n,
@@ -692,6 +901,43 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache,
   DNET_CHECK(lds <= 160 * 1024, "attn_mod: head sizes exceed LDS");
   const dim3 grid((unsigned)((T + P.QT - 1) / P.QT), (unsigned)(Hkv * GS),
                   (unsigned)B);
+  // bf16 decode with many heads per kv head: the grouped heads are the rows
+  // of the matrix-core tile (the Python side sizes `partials` by the same
+  // rule: attn_mod_heads_on_mfma)
+  if (!f32 && T == 1 && G >= kHeadsMfmaMinGroup && pool == 0 && D % 8 == 0 &&
+      DV % 8 == 0) {
+    const int ns = (int)std::max<int64_t>(1, splits);
+    DNET_CHECK(partials.has_value() &&
+                   partials->scalar_type() == torch::kFloat32 &&
+                   partials->is_contiguous() &&
+                   partials->numel() >= B * Hq * ns * (int64_t)(DV + 2),
+               "partials fp32 [B, Hq, splits, DV+2]");
+    float* part = partials->data_ptr<float>();
+    const int GT = (G + 63) / 64;
+    const dim3 hgrid((unsigned)ns, (unsigned)(Hkv * GT), (unsigned)B);
+#define AH(DCC, NVV)                                                         \
+  hipLaunchKernelGGL((attn_mod_mfma_heads<DCC, NVV>), hgrid, dim3(256), 0,   \
+                     stream, (const short*)q.data_ptr(),                     \
+                     (const short*)kcache.data_ptr(),                        \
+                     (const short*)vcache.data_ptr(), part, ns, P)
+#define AH_V(DCC)                          \
+  do {                                     \
+    if (DV <= 64) AH(DCC, 4);              \
+    else if (DV <= 128) AH(DCC, 8);        \
+    else if (DV <= 192) AH(DCC, 12);       \
+    else AH(DCC, 16);                      \
+  } while (0)
+    if (D <= 64) AH_V(2);
+    else if (D <= 128) AH_V(4);
+    else if (D <= 192) AH_V(6);
+    else AH_V(8);
+#undef AH_V
+#undef AH
+    hipLaunchKernelGGL((attn_mod_combine<short>), dim3((unsigned)(B * Hq)),
+                       dim3(64), 0, stream, part, (short*)out.data_ptr(),
+                       P.sinks, P.pos, P.slots, Hq, DV, ns, Bc);
+    return;
+  }
   // bf16 prompts: matrix-core kernel (head sizes padded to its tile classes)
   if (!f32 && T >= 16 && D % 8 == 0 && DV % 8 == 0) {
     const dim3 mgrid((unsigned)((T + 63) / 64), (unsigned)Hq, (unsigned)B);

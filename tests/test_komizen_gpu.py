@@ -176,20 +176,62 @@ def test_model_gpu_matches_cpu(dtype):
     g = torch.Generator().manual_seed(5)
     prompts = [torch.randint(0, 160, (n,), generator=g) for n in (70, 9)]
     want = [[0, 33, 69], [8]]
-    tol = dict(atol=2e-3, rtol=2e-3) if dtype == "float32" \
-        else dict(atol=0.25, rtol=0.1)
+
+    def same(y, x):
+        # float32 is the sharp comparison; in bfloat16 the two paths round
+        # differently and these random stacks multiply that noise layer by
+        # layer, so the bound is on the root mean square
+        y, x = y.float().cpu(), x.float()
+        if dtype == "float32":
+            torch.testing.assert_close(y, x, atol=2e-3, rtol=2e-3)
+        else:
+            rel = float((y - x).pow(2).mean().sqrt() / x.pow(2).mean().sqrt())
+            assert rel < 0.3, rel
+
     a = cpu.prefill_slots([2, 0], prompts, want=want)
     b = gpu.prefill_slots([2, 0], prompts, want=want)
     for x, y in zip(a, b):
-        torch.testing.assert_close(y.float().cpu(), x.float(), **tol)
+        same(y, x)
     park = torch.tensor([False, True, False])
     for step in range(4):
         toks = torch.randint(0, 160, (3,), generator=g)
         for ex in (cpu, gpu):
             ex.tokbuf[0].copy_(toks)
             ex.slot_step_compute(park=park.to(ex.device))
-        torch.testing.assert_close(
-            gpu.logits_buf[0].float().cpu()[[0, 2]],
-            cpu.logits_buf[0].float()[[0, 2]], **tol)
+        same(gpu.logits_buf[0][[0, 2]], cpu.logits_buf[0][[0, 2]])
         for ex in (cpu, gpu):
             ex.kvs[0].pos.add_((~park).to(ex.device).to(torch.int32))
+
+
+@pytest.mark.parametrize("Hq,Hkv,D,DV,share", [
+    (32, 1, 256, 192, True), (20, 1, 160, 128, True), (80, 1, 72, 40, True),
+    (32, 2, 64, 64, False), (48, 1, 128, 128, False)])
+@pytest.mark.parametrize("window", [0, 50])
+def test_decode_heads_on_matrix_cores(Hq, Hkv, D, DV, share, window):
+    """bf16 decode with >= 16 heads per kv head: the grouped heads share the
+    staged key tiles on the matrix cores; split over the keys, every score
+    modifier, idle rows, slot indirection, positions at tile borders."""
+    torch.manual_seed(Hq + D)
+    B, Bc, S = 5, 6, 320
+    dt = torch.bfloat16
+    kc = torch.randn(Bc, Hkv, S, D, device=DEV).to(dt)
+    vc = None if share else torch.randn(Bc, Hkv, S, DV, device=DEV).to(dt)
+    q = (torch.randn(B, Hq * D, device=DEV) * 0.5).to(dt)
+    pos = _i32([0, 31, 32, 300, 77])
+    lens = _i32([1, 1, 1, 1, 0])
+    slots = _i32([5, 0, 3, 1, 2])
+    temp = torch.rand(Hq, device=DEV) + 0.5
+    r1, r2 = torch.rand(Hq, device=DEV) * 0.3, torch.rand(Hq, device=DEV)
+    sinks = torch.randn(Hq, device=DEV)
+    for mods in (dict(), dict(temp=temp, softcap=5.0, dist_r1=r1, dist_r2=r2,
+                              sinks=sinks)):
+        out = ops.attn_mod(q, kc, vc, pos.to(DEV), 1, D ** -0.5,
+                           lens.to(DEV), slots.to(DEV), window=window,
+                           v_dim=DV if share else 0, **mods)
+        cm = {k: (v.cpu() if torch.is_tensor(v) else v)
+              for k, v in mods.items()}
+        want = ref.attn_mod(q.cpu(), kc.cpu(), None if share else vc.cpu(),
+                            pos, 1, D ** -0.5, lens, slots, window=window,
+                            v_dim=DV if share else 0, **cm)
+        torch.testing.assert_close(out.cpu().float()[:4], want.float()[:4],
+                                   atol=3e-2, rtol=3e-2)
