@@ -425,10 +425,8 @@ class KomizenRingModel(RingModel):
         T = u.shape[0]
         W = self.cfg.hidden_size
         E, top = int(ff["router"]["experts"]), int(ff["router"]["top"])
-        probs = torch.softmax(lw.router(u.float()), dim=-1)
-        val, idx = torch.topk(probs, top, dim=-1)
-        we = torch.zeros(T, E, dtype=torch.float32, device=u.device)
-        we.scatter_(1, idx, val * float(ff["router"]["scale"]))
+        we = ops.moe_route(lw.router(u.float()), top,
+                           float(ff["router"]["scale"]))
         I = lw.up_w.shape[1]
         if (T * top < E and self.wdtype == torch.bfloat16
                 and W % 8 == 0 and I % 8 == 0):
@@ -447,7 +445,7 @@ class KomizenRingModel(RingModel):
                           lw.up_w.transpose(1, 2))              # [E, T, I]
             a = ops.act_slice(z.view(E * T, I), 0, I, "relu_sq")
             d = torch.bmm(a.view(E, T, I), lw.down_w.transpose(1, 2))
-            return torch.einsum("te,etw->tw", we, d.float())
+            return ops.moe_weighted_sum(d, we)
         out = torch.zeros(T, W, dtype=torch.float32, device=u.device)
         hit = (we > 0).any(dim=0).tolist()
         for e in range(E):

@@ -758,3 +758,22 @@ def moe_up_act(x, w, we) -> torch.Tensor:
         _native().moe_up_act(x, w, we, act)
         return act
     return ref.moe_up_act(x, w, we)
+
+
+def moe_route(logits, top: int, scale: float) -> torch.Tensor:
+    """Routing weights [T, E]: softmax over all experts, the ``top`` largest
+    kept times ``scale``, not renormalized (one kernel; no host sync)."""
+    if logits.is_cuda:
+        we = torch.empty_like(logits)
+        _native().moe_route(logits.contiguous(), we, top, scale)
+        return we
+    return ref.moe_route(logits, top, scale)
+
+
+def moe_weighted_sum(d, we) -> torch.Tensor:
+    if d.is_cuda and d.shape[2] % 4 == 0:
+        out = torch.empty(d.shape[1], d.shape[2], dtype=torch.float32,
+                          device=d.device)
+        _native().moe_weighted_sum(d.contiguous(), we, out)
+        return out
+    return ref.moe_weighted_sum(d, we)

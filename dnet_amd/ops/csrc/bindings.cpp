@@ -154,6 +154,9 @@ void latent_q_pack(torch::Tensor q, torch::Tensor qabs, torch::Tensor rot_freq,
                    int64_t d);
 void moe_up_act(torch::Tensor x, torch::Tensor w, torch::Tensor we,
                 torch::Tensor act);
+void moe_route(torch::Tensor logits, torch::Tensor we, int64_t top,
+               double scale);
+void moe_weighted_sum(torch::Tensor d, torch::Tensor we, torch::Tensor out);
 }  // namespace dnet
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -244,4 +247,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "latent attention: queries in the cache row's layout");
   m.def("moe_up_act", &dnet::moe_up_act,
         "grouped ungated expert up projection + squared ReLU");
+  m.def("moe_route", &dnet::moe_route,
+        "softmax over all experts, top-k kept, scaled, not renormalized");
+  m.def("moe_weighted_sum", &dnet::moe_weighted_sum,
+        "sum over experts of routing weight times expert result");
 }

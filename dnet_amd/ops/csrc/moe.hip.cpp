@@ -350,6 +350,76 @@ __global__ __launch_bounds__(256, 4) void moe_down_kernel(
   }
 }
 
+// ---- routing and merging for batched expert products -----------------------
+// moe_route: we[t, e] = softmax(logits[t, :])[e] * scale for the `top`
+// largest probabilities of row t, 0 elsewhere (the weights are not
+// renormalized; ties go to the lower index). One thread per row; fp32 with
+// the accurate expf.
+__global__ __launch_bounds__(256) void moe_route_kernel(
+    const float* __restrict__ logits, float* __restrict__ we, const int T,
+    const int E, const int top, const float scale) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  const float* lr = logits + (int64_t)t * E;
+  float* wr = we + (int64_t)t * E;
+  float mx = lr[0];
+  for (int e = 1; e < E; ++e) mx = fmaxf(mx, lr[e]);
+  float sum = 0.f;
+  for (int e = 0; e < E; ++e) {
+    const float p = expf(lr[e] - mx);
+    wr[e] = -p;                 // negative: not chosen yet
+    sum += p;
+  }
+  const float k = scale / sum;
+  for (int c = 0; c < top; ++c) {
+    int best = -1;
+    float bp = 0.f;
+    for (int e = 0; e < E; ++e) {
+      const float p = -wr[e];
+      if (p > bp) {             // chosen entries are >= 0 and never win
+        bp = p;
+        best = e;
+      }
+    }
+    if (best < 0) break;
+    wr[best] = bp * k;
+  }
+  for (int e = 0; e < E; ++e)
+    if (wr[e] < 0.f) wr[e] = 0.f;
+}
+
+// moe_weighted_sum: out[t, :] = sum_e we[t, e] * d[e, t, :] (fp32 sum of the
+// experts' results as they come out of the batched product).
+template <typename T>
+__global__ __launch_bounds__(256) void moe_weighted_sum_kernel(
+    const T* __restrict__ d, const float* __restrict__ we,
+    float* __restrict__ out, const int Tn, const int E, const int W) {
+  const int t = blockIdx.y;
+  const int w = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (w >= W) return;
+  float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+  for (int e = 0; e < E; ++e) {
+    const float c = we[(int64_t)t * E + e];
+    if (c == 0.f) continue;
+    const T* dp = d + ((int64_t)e * Tn + t) * W + w;
+    if constexpr (sizeof(T) == 2) {
+      const short4v v = *reinterpret_cast<const short4v*>(dp);
+      a0 = fmaf(c, bits2f(v.x[0]), a0);
+      a1 = fmaf(c, bits2f(v.x[1]), a1);
+      a2 = fmaf(c, bits2f(v.x[2]), a2);
+      a3 = fmaf(c, bits2f(v.x[3]), a3);
+    } else {
+      const float4 v = *reinterpret_cast<const float4*>(dp);
+      a0 = fmaf(c, v.x, a0);
+      a1 = fmaf(c, v.y, a1);
+      a2 = fmaf(c, v.z, a2);
+      a3 = fmaf(c, v.w, a3);
+    }
+  }
+  *reinterpret_cast<float4*>(out + (int64_t)t * W + w) =
+      make_float4(a0, a1, a2, a3);
+}
+
 template <typename LaunchFn>
 static void moe_dispatch_m(int M, LaunchFn&& fn) {
   switch (M) {
@@ -488,6 +558,43 @@ void moe_up_act(torch::Tensor x, torch::Tensor w, torch::Tensor we,
     });
     m0 += mt;
   }
+}
+
+void moe_route(torch::Tensor logits, torch::Tensor we, int64_t top,
+               double scale) {
+  DNET_CHECK(logits.dim() == 2 && logits.scalar_type() == torch::kFloat &&
+                 logits.is_contiguous() && we.scalar_type() == torch::kFloat &&
+                 we.is_contiguous() && we.sizes() == logits.sizes(),
+             "moe_route: logits, we fp32 [T, E]");
+  const int64_t T = logits.size(0), E = logits.size(1);
+  DNET_CHECK(E >= 1 && top >= 1 && top <= E, "moe_route: 1 <= top <= E");
+  if (T == 0) return;
+  hipLaunchKernelGGL(moe_route_kernel, dim3(cdiv(T, 256)), dim3(256), 0,
+                     current_stream(), logits.data_ptr<float>(),
+                     we.data_ptr<float>(), (int)T, (int)E, (int)top,
+                     (float)scale);
+}
+
+void moe_weighted_sum(torch::Tensor d, torch::Tensor we, torch::Tensor out) {
+  DNET_CHECK(d.dim() == 3 && d.is_contiguous() && we.is_contiguous() &&
+                 we.scalar_type() == torch::kFloat && out.is_contiguous() &&
+                 out.scalar_type() == torch::kFloat, "moe_weighted_sum args");
+  const int64_t E = d.size(0), T = d.size(1), W = d.size(2);
+  DNET_CHECK(we.size(0) == T && we.size(1) == E && out.size(0) == T &&
+                 out.size(1) == W && W % 4 == 0, "moe_weighted_sum shapes");
+  if (T == 0) return;
+  const dim3 grid(cdiv(W / 4, 256), (unsigned)T);
+  auto st = current_stream();
+  if (d.scalar_type() == torch::kBFloat16)
+    hipLaunchKernelGGL((moe_weighted_sum_kernel<short>), grid, dim3(256), 0,
+                       st, (const short*)d.data_ptr(), we.data_ptr<float>(),
+                       out.data_ptr<float>(), (int)T, (int)E, (int)W);
+  else if (d.scalar_type() == torch::kFloat)
+    hipLaunchKernelGGL((moe_weighted_sum_kernel<float>), grid, dim3(256), 0,
+                       st, d.data_ptr<float>(), we.data_ptr<float>(),
+                       out.data_ptr<float>(), (int)T, (int)E, (int)W);
+  else
+    DNET_CHECK(false, "moe_weighted_sum: dtype");
 }
 
 void moe_down(torch::Tensor act, torch::Tensor w,

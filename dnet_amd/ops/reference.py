@@ -1031,3 +1031,19 @@ def moe_up_act(x: torch.Tensor, w: torch.Tensor, we: torch.Tensor
     hold anything; ``moe_down`` never reads them)."""
     z = torch.einsum("mk,eik->emi", x.float(), w.float())
     return (torch.relu(z) ** 2).to(torch.bfloat16)
+
+
+def moe_route(logits: torch.Tensor, top: int, scale: float) -> torch.Tensor:
+    """Routing weights [T, E] fp32: softmax over all experts, the ``top``
+    largest probabilities kept and multiplied by ``scale`` (not
+    renormalized), 0 for the rest."""
+    probs = torch.softmax(logits.float(), dim=-1)
+    val, idx = torch.topk(probs, top, dim=-1)
+    we = torch.zeros_like(probs)
+    we.scatter_(1, idx, val * scale)
+    return we
+
+
+def moe_weighted_sum(d: torch.Tensor, we: torch.Tensor) -> torch.Tensor:
+    """d [E, T, W], we [T, E] -> fp32 [T, W] = sum_e we[t, e] d[e, t]."""
+    return torch.einsum("te,etw->tw", we.float(), d.float())

@@ -235,3 +235,20 @@ def test_decode_heads_on_matrix_cores(Hq, Hkv, D, DV, share, window):
                             v_dim=DV if share else 0, **cm)
         torch.testing.assert_close(out.cpu().float()[:4], want.float()[:4],
                                    atol=3e-2, rtol=3e-2)
+
+
+@pytest.mark.parametrize("T,E,top", [(1, 8, 4), (33, 5, 2), (700, 64, 6),
+                                     (4, 3, 3), (9, 16, 1)])
+def test_route_and_weighted_sum(T, E, top):
+    torch.manual_seed(T + E)
+    logits = torch.randn(T, E, device=DEV) * 2
+    we = ops.moe_route(logits, top, 1.5)
+    want = ref.moe_route(logits.cpu(), top, 1.5)
+    torch.testing.assert_close(we.cpu(), want, atol=1e-6, rtol=1e-5)
+    assert int((we > 0).sum(1).min()) == top == int((we > 0).sum(1).max())
+    for dt in DTS:
+        d = torch.randn(E, T, 72, device=DEV).to(dt)
+        out = ops.moe_weighted_sum(d, we)
+        torch.testing.assert_close(out.cpu(),
+                                   ref.moe_weighted_sum(d.cpu(), want),
+                                   atol=1e-4, rtol=1e-4)
