@@ -96,16 +96,25 @@ class KomizenRingModel(RingModel):
                                   device=self.device)
         for lid in self.layer_ids:
             s = self._spec(lid)
-            if s["type"] == "latent_attention":
+            if s["type"] == "latent_attention" and not self._latent_fits(
+                    s["mixer"]):
                 m = s["mixer"]
-                if m["kv_rank"] + m["rot_dim"] > self.MAX_LATENT_ROW:
+                if max(m["dim"] + m["rot_dim"], m["vdim"]) \
+                        > self.MAX_LATENT_ROW:
                     raise NotImplementedError(
-                        f"komizen layer run {lid}: kv_rank + rot_dim = "
-                        f"{m['kv_rank'] + m['rot_dim']} exceeds the attention "
-                        f"kernels' row of {self.MAX_LATENT_ROW}")
+                        f"komizen layer run {lid}: neither the latent row "
+                        f"({m['kv_rank'] + m['rot_dim']}) nor the per-head "
+                        f"key / value sizes fit the attention kernels' row "
+                        f"of {self.MAX_LATENT_ROW}")
 
     def _init_positional(self):
         pass        # angles are computed from positions inside the kernels
+
+    def _latent_fits(self, m: dict) -> bool:
+        """Whether the shared row [latent | rotated key part] fits one key
+        row of the attention kernels. If not, the layer caches per-head keys
+        and values instead (same kernels, a larger cache)."""
+        return m["kv_rank"] + m["rot_dim"] <= self.MAX_LATENT_ROW
 
     @property
     def hidden_width(self) -> int:
@@ -137,7 +146,11 @@ class KomizenRingModel(RingModel):
             m = s["mixer"]
             taps = max(int(m.get("conv") or 1) - 1, 0)
             if s["type"] == "latent_attention":
-                dims.append((1, m["kv_rank"] + m["rot_dim"], 0))
+                if self._latent_fits(m):
+                    dims.append((1, m["kv_rank"] + m["rot_dim"], 0))
+                else:
+                    dims.append((m["heads"], m["dim"] + m["rot_dim"],
+                                 m["vdim"]))
                 states.append({})
             elif s["type"] == "delta":
                 H, KH, d, dv, C = self._delta_dims(m)
@@ -202,6 +215,8 @@ class KomizenRingModel(RingModel):
                 .contiguous()
             lw.uv = uv.to(self.wdtype).to(self.device).view(H, dv, R) \
                 .transpose(1, 2).contiguous()
+            if not self._latent_fits(m):
+                lw.kv_b = self._lin(torch.cat([uk, uv]))    # [uk ; uv]
             lw.o = self._lin(get("mix.o"))
             n = int(m["rot"]["dims"])
             f = [float(m["rot"]["base"]) ** (-2.0 * i / n)
@@ -383,6 +398,9 @@ class KomizenRingModel(RingModel):
         cq = ops.rmsnorm_rows(p[:, :QR], lw.q_a_norm, self.cfg.rms_eps,
                               self.wdtype)
         q = lw.q_b(cq)                                 # [M, H*(d+rd)]
+        if kv.v[li] is not None:
+            return self._expanded_attention(p, q, lw, m, kv, li, pos, T,
+                                            lens, slots)
         ops.latent_append(p, QR, lw.kv_a_norm, self.cfg.rms_eps, R,
                           lw.rot_freq, kv.k[li], pos, T, lens, slots)
         # plain query part into the latent space, head by head
@@ -393,6 +411,40 @@ class KomizenRingModel(RingModel):
                           lens, slots, v_dim=R)        # [M, H*R]
         ov = torch.bmm(ol.view(M, H, R).transpose(0, 1), lw.uv)
         return lw.o(ov.transpose(0, 1).reshape(M, H * dv))
+
+    def _expanded_attention(self, p, q, lw, m, kv, li, pos, T, lens, slots):
+        """Latent rows too wide for one key row of the kernels: per-head keys
+        [plain | rotated shared part] and values are formed from the latent
+        and cached. Padding and idle rows write where their slot's next real
+        token is written later, before anything reads it."""
+        H, d, rd, dv = m["heads"], m["dim"], m["rot_dim"], m["vdim"]
+        R, QR = m["kv_rank"], m["q_rank"]
+        M = p.shape[0]
+        B = M // T
+        c = ops.rmsnorm_rows(p[:, QR:QR + R], lw.kv_a_norm, self.cfg.rms_eps,
+                             self.wdtype)
+        kvu = lw.kv_b(c)                               # [ku (H*d) | v (H*dv)]
+        ku = kvu[:, :H * d].reshape(M, H, d)
+        kin = torch.cat([ku, p[:, QR + R:QR + R + rd].reshape(M, 1, rd)
+                         .expand(M, H, rd)], dim=-1).reshape(M, H * (d + rd))
+        # the rotation kernel of the query pack turns the rotated parts and
+        # copies the plain ones
+        k = ops.latent_q_pack(kin.contiguous(),
+                              ku.transpose(0, 1).contiguous(), lw.rot_freq,
+                              pos, T, H, d)
+        qr = ops.latent_q_pack(
+            q, q.view(M, H, d + rd)[:, :, :d].transpose(0, 1).contiguous(),
+            lw.rot_freq, pos, T, H, d)
+        smax = kv.k[li].shape[2]
+        at = (pos.view(B, 1).long()
+              + torch.arange(T, device=p.device)).clamp_(max=smax - 1)
+        sl = (slots.long() if slots is not None
+              else torch.arange(B, device=p.device)).view(B, 1)
+        kv.k[li][sl, :, at] = k.view(B, T, H, d + rd)
+        kv.v[li][sl, :, at] = kvu[:, H * d:].reshape(B, T, H, dv)
+        a = ops.attn_mod(qr, kv.k[li], kv.v[li], pos, T, float(m["scale"]),
+                         lens, slots)
+        return lw.o(a)
 
     def _delta(self, u, lw, m, kv, li, pos, T, lens, slots):
         H, KH, d, dv, C = self._delta_dims(m)

@@ -34,7 +34,7 @@ def base_cfg(**kw):
                 delta_heads=4, delta_kv_heads=2, delta_dim=8, delta_vdim=12,
                 ssm_heads=6, ssm_vdim=4, ssm_state=8, ssm_groups=2,
                 norm_groups=3, conv=3, experts=5, top=2, expert_ff=24,
-                router_scale=1.5, embedding_scale=3.0, rot_base=300.0)
+                router_scale=1.25, embedding_scale=3.0, rot_base=300.0)
     args.update(kw)
     cfg = komizen_config(48, V, **args)
     cfg["layers"] = copy.deepcopy(cfg["layers"])
@@ -432,6 +432,34 @@ def test_other_sizes(device, kw):
         close(lg[1:2], wb[4 + i].view(1, -1))
 
 
+@pytest.mark.parametrize("device", DEVICES)
+def test_latent_row_wider_than_the_kernels_key_row(device, monkeypatch):
+    """When the shared latent row does not fit one key row of the attention
+    kernels the layer caches per-head keys and values: same logits, through
+    ragged prompts, portions, batched decode with an idle row."""
+    from dnet_amd.models import KomizenRingModel
+    monkeypatch.setattr(KomizenRingModel, "MAX_LATENT_ROW", 24)
+    cfg = base_cfg()                        # latent row 24 + 8 = 32 > 24
+    sd = O.make_checkpoint(cfg, 13)
+    a, b = tokens(33, 11), tokens(6, 12)
+    wa, wb = oracle(a, cfg, sd), oracle(b, cfg, sd)
+    ex = executor(cfg, sd, device, slots=3)
+    assert ex.kvs[0].v[0] is not None and ex.kvs[0].k[0].shape[1] == 3
+    got = ex.prefill_slots([2, 0], [a[:25], b[:3]],
+                           want=[list(range(25)), [2]], chunk=7)
+    close(got[0], wa[:25])
+    close(got[1], wb[2:3])
+    for i in range(3):
+        lg = decode_step(ex, {2: a[25 + i], 0: b[3 + i]})
+        close(lg[2:3], wa[25 + i].view(1, -1))
+        close(lg[0:1], wb[3 + i].view(1, -1))
+    for i in range(28, 33):
+        close(decode_step(ex, {2: a[i]})[2:3], wa[i].view(1, -1))
+    with pytest.raises(NotImplementedError):
+        monkeypatch.setattr(KomizenRingModel, "MAX_LATENT_ROW", 8)
+        executor(cfg, sd, device)
+
+
 @pytest.mark.gpu
 def test_decode_graph_replays_match_eager():
     """Captured decode steps, replayed with eager prefills and host syncs in
@@ -636,21 +664,27 @@ def test_two_stage_ring_matches_single():
     tokens equal the single-stage run."""
     import multiprocessing as mp
     import socket
-    single = _ring_run(0, 1)
-    s = socket.socket()
-    s.bind(("127.0.0.1", 0))
-    port = s.getsockname()[1]
-    s.close()
     ctx = mp.get_context("spawn")
-    q = ctx.Queue()
-    procs = [ctx.Process(target=_ring_rank_main, args=(r, 2, port, q))
-             for r in range(2)]
-    for p in procs:
-        p.start()
-    out = q.get(timeout=200)
-    for p in procs:
-        p.join(timeout=60)
-        assert p.exitcode == 0
+
+    def run(world):
+        # the single-stage run is spawned too: same thread settings and
+        # library state as the ranks, so equal tokens mean equal arithmetic
+        s = socket.socket()
+        s.bind(("127.0.0.1", 0))
+        port = s.getsockname()[1]
+        s.close()
+        q = ctx.Queue()
+        procs = [ctx.Process(target=_ring_rank_main, args=(r, world, port, q))
+                 for r in range(world)]
+        for p in procs:
+            p.start()
+        out = q.get(timeout=200)
+        for p in procs:
+            p.join(timeout=60)
+            assert p.exitcode == 0
+        return out
+
+    single, out = run(1), run(2)
     assert single.shape[0] == 2 and single.shape[1] >= 6
     assert torch.equal(out, single)
 
