@@ -175,6 +175,46 @@ def _executors(dtype, mb=3, smax=192):
 
 
 @pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_odd_sizes_gpu_matches_cpu(dtype):
+    """Sizes that are multiples of nothing (width, vocabulary, ranks, head
+    sizes, expert width): every kernel's unvectorized path and the linears'
+    fallbacks, prompt and decode."""
+    from dnet_amd.models import ModelConfig
+    from dnet_amd.models.config import komizen_config
+    from dnet_amd.parallel.ring import RingExecutor
+    from komizen_oracle import make_checkpoint
+    hf = komizen_config(52, 77, "ldm", layers=3, streams=3, heads=3, dim=10,
+                        rot_dim=6, vdim=14, kv_rank=18, q_rank=11,
+                        delta_heads=3, delta_kv_heads=3, delta_dim=5,
+                        delta_vdim=7, ssm_heads=2, ssm_vdim=9, ssm_state=5,
+                        ssm_groups=1, norm_groups=1, conv=2, experts=3, top=2,
+                        expert_ff=13, router_scale=0.8, embedding_scale=2.0)
+    sd = make_checkpoint(hf, seed=21,
+                         ff_gain=1.0 if dtype == "float32" else 0.1)
+    g = torch.Generator().manual_seed(6)
+    prompts = [torch.randint(0, 77, (n,), generator=g) for n in (19, 3)]
+    outs = []
+    for dev, graphs in (("cpu", False), (DEV, True)):
+        cfg = ModelConfig.from_hf(hf)
+        cfg.compute_dtype = dtype
+        ex = RingExecutor(cfg, 0, 1, torch.device(dev), mb_size=2, smax=64,
+                          use_graphs=graphs, init_weights=False)
+        ex.model.load_state_dict(sd)
+        rows = [r.float().cpu() for r in ex.prefill_slots(
+            [1, 0], prompts, want=[list(range(19)), [2]])]
+        for step in range(3):
+            ex.tokbuf[0].copy_(torch.tensor([5 + step, 9 + step]))
+            ex.slot_step_compute(park=torch.zeros(2, dtype=torch.bool,
+                                                  device=ex.device))
+            rows.append(ex.logits_buf[0].float().cpu().clone())
+            ex.kvs[0].pos.add_(1)
+        outs.append(torch.cat(rows))
+    cpu, gpu = outs
+    rel = float((gpu - cpu).pow(2).mean().sqrt() / cpu.pow(2).mean().sqrt())
+    assert rel < (2e-4 if dtype == "float32" else 0.2), rel
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
 def test_model_gpu_matches_cpu(dtype):
     """Ragged prefill into slots, then graph-captured decode steps with one
     row idle, on the GPU kernels against the CPU reference ops."""
