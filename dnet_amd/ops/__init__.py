@@ -683,7 +683,8 @@ def clamped_glu(gu: torch.Tensor, alpha: float, limit: float) -> torch.Tensor:
 
 
 # ---- residual streams, gated delta rule, latent attention (komizen) ----
-# csrc/streams.hip.cpp, csrc/gated_delta.hip.cpp, csrc/latent.hip.cpp. The
+# csrc/streams.hip.cpp, csrc/seq_state.hip.cpp (gated_delta_scan),
+# csrc/latent.hip.cpp, csrc/attn_mod.hip.cpp, csrc/moe.hip.cpp. The
 # streams, the recurrent state, unit norms, decays and angles are fp32
 # whatever the activation dtype.
 

@@ -67,8 +67,16 @@ __global__ __launch_bounds__(256) void hc_write_read_kernel(
     for (int j = 0; j < VW; ++j) u[j] = 0.f;
     if (yr) {
       float yv[VW];
+      if constexpr (VW == 4 && sizeof(TY) == 4) {
+        const float4 v = *reinterpret_cast<const float4*>(yr + i);
+        yv[0] = v.x; yv[1] = v.y; yv[2] = v.z; yv[3] = v.w;
+      } else if constexpr (VW == 4) {
+        const short4v v = *reinterpret_cast<const short4v*>(yr + i);
 #pragma unroll
-      for (int j = 0; j < VW; ++j) yv[j] = ldf<TY>(yr + i + j);
+        for (int j = 0; j < 4; ++j) yv[j] = bits2f(v.x[j]);
+      } else {
+        yv[0] = ldf<TY>(yr + i);
+      }
 #pragma unroll
       for (int t = 0; t < kMaxStreams; ++t)
         if (t < S) {
@@ -119,12 +127,32 @@ __global__ __launch_bounds__(256) void hc_write_read_kernel(
     for (int t = 0; t < kMaxStreams; ++t)
       if (t < S) {
         const float ci = sw.in[t];
-#pragma unroll
-        for (int j = 0; j < VW; ++j)
-          u[j] = fmaf(ci, xr[(int64_t)t * W + i + j], u[j]);
+        if constexpr (VW == 4) {
+          const float4 v =
+              *reinterpret_cast<const float4*>(xr + (int64_t)t * W + i);
+          u[0] = fmaf(ci, v.x, u[0]);
+          u[1] = fmaf(ci, v.y, u[1]);
+          u[2] = fmaf(ci, v.z, u[2]);
+          u[3] = fmaf(ci, v.w, u[3]);
+        } else {
+          u[0] = fmaf(ci, xr[(int64_t)t * W + i], u[0]);
+        }
       }
-#pragma unroll
-    for (int j = 0; j < VW; ++j) stf<TO>(orow + i + j, u[j] * r * wn[i + j]);
+    if constexpr (VW == 4) {
+      const float4 g = *reinterpret_cast<const float4*>(wn + i);
+      const float o0 = u[0] * r * g.x, o1 = u[1] * r * g.y;
+      const float o2 = u[2] * r * g.z, o3 = u[3] * r * g.w;
+      if constexpr (sizeof(TO) == 4) {
+        *reinterpret_cast<float4*>(orow + i) = make_float4(o0, o1, o2, o3);
+      } else {
+        short4v pk;
+        pk.x[0] = f2bits(o0); pk.x[1] = f2bits(o1);
+        pk.x[2] = f2bits(o2); pk.x[3] = f2bits(o3);
+        *reinterpret_cast<short4v*>(orow + i) = pk;
+      }
+    } else {
+      stf<TO>(orow + i, u[0] * r * wn[i]);
+    }
   }
 }
 
