@@ -265,6 +265,8 @@ class ModelConfig:
             num_experts=max((m["router"]["experts"] for m in moe), default=0),
             num_experts_per_tok=max((m["router"]["top"] for m in moe),
                                     default=0),
+            moe_intermediate_size=max((m["expert"]["ff"] for m in moe),
+                                      default=0),
             vocab_size=cfg["vocab"],
             rms_eps=cfg["norm"]["eps"],
             embedding_scale=float((cfg.get("embedding") or {}).get("scale",

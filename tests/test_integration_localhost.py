@@ -191,3 +191,36 @@ def test_sequence_state_family_over_two_shards(cluster):
         assert texts[0] == texts[1]
         r = c.post(f"{api}/v1/unload_model")
         assert r.status_code == 200
+
+
+@pytest.mark.timeout(300)
+def test_looped_multi_stream_family_over_two_shards(cluster):
+    """A family with several residual streams and a looped layer span
+    (komizen: 4 stored layers, 6 layer runs) split over the two shards in the
+    middle of the loop: both shards load the looped layers' tensors, all
+    streams ride the hops, chats complete and repeat."""
+    api = cluster["api"]
+    name = "komizen-tiny-random"
+    with httpx.Client(timeout=180) as c:
+        r = c.post(f"{api}/v1/prepare_topology_manual", json={
+            "model": name,
+            "assignments": [
+                {"instance": "shard0", "layers": [0, 1, 2]},
+                {"instance": "shard1", "layers": [3, 4, 5]}]})
+        assert r.status_code == 200, r.text
+        r = c.post(f"{api}/v1/load_model",
+                   json={"model": name, "max_tokens": 8})
+        assert r.status_code == 200, r.text
+        texts = []
+        for _ in range(2):          # greedy: the same prompt repeats exactly
+            r = c.post(f"{api}/v1/chat/completions", json={
+                "model": name, "stream": False, "max_tokens": 8,
+                "temperature": 0.0,
+                "messages": [{"role": "user", "content": "loop please"}]})
+            assert r.status_code == 200, r.text
+            body = r.json()
+            assert body["usage"]["completion_tokens"] >= 1
+            texts.append(body["choices"][0]["message"]["content"])
+        assert texts[0] == texts[1]
+        r = c.post(f"{api}/v1/unload_model")
+        assert r.status_code == 200
