@@ -20,7 +20,9 @@ Mixers (``cfg.layer_specs[run]["type"]``):
   space: each head's plain query part is carried through its key
   up-projection first, the scores are taken against the cached rows, the
   softmax-weighted sum of the latents is carried through the head's value
-  up-projection afterwards. Nothing per head is ever cached.
+  up-projection afterwards. Nothing per head is cached (unless the shared
+  row is wider than the attention kernels' key row: then per-head keys and
+  values are, see ``_expanded_attention``).
 * ``delta``: gated delta rule. q/k/v pass short causal convolutions + SiLU;
   q, k are made unit vectors per head; per value head
   S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q, then a per-head
@@ -175,9 +177,9 @@ class KomizenRingModel(RingModel):
         # small per-channel / per-head parameters feed fp32 math directly
         return t.to(torch.float32).to(self.device).contiguous()
 
-    def _build_layer(self, spec: dict, get, has) -> LayerWeights:
+    def _build_layer(self, spec: dict, get) -> LayerWeights:
         """Weights of one stored layer. ``get(name)`` returns the tensor
-        ``l<i>.<name>``; ``has(name)`` tells whether it exists."""
+        ``l<i>.<name>``."""
         m = spec["mixer"]
         W = self.cfg.hidden_size
         S = self.streams
@@ -279,8 +281,7 @@ class KomizenRingModel(RingModel):
 
     def load_state_dict(self, sd: dict):
         self._bind_runs(lambda wid, spec: self._build_layer(
-            spec, lambda n, p=f"l{wid}.": sd[p + n],
-            lambda n, p=f"l{wid}.": (p + n) in sd))
+            spec, lambda n, p=f"l{wid}.": sd[p + n]))
         if self.is_first or self.is_last:
             emb = sd["embed"].to(self.wdtype).to(self.device).contiguous()
             if self.is_first:
@@ -367,7 +368,7 @@ class KomizenRingModel(RingModel):
                 for e in range(ff["router"]["experts"]):
                     t[f"mlp.e{e}.up"] = lin(g, ef, W)
                     t[f"mlp.e{e}.down"] = lin(g, W, ef)
-            return self._build_layer(spec, t.__getitem__, t.__contains__)
+            return self._build_layer(spec, t.__getitem__)
 
         self._bind_runs(build)
         if self.is_first or self.is_last:
