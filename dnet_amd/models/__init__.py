@@ -51,5 +51,9 @@ from .komizen import KomizenRingModel  # noqa: E402
 
 register(KomizenRingModel)
 
-__all__ = ["GegoraxRingModel", "KomizenRingModel", "ModelConfig", "QuantConfig", "RingModel", "MoERingModel", "KVCache", "PosudraRingModel",
+from .lurisun import LurisunRingModel  # noqa: E402
+
+register(LurisunRingModel)
+
+__all__ = ["GegoraxRingModel", "KomizenRingModel", "LurisunRingModel", "ModelConfig", "QuantConfig", "RingModel", "MoERingModel", "KVCache", "PosudraRingModel",
            "Linear", "PRESETS", "get_ring_model", "register"]

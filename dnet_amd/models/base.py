@@ -284,7 +284,8 @@ class KVCache:
                  smax: int, device, kv_bits: int = 16,
                  layer_dims: Optional[Sequence[tuple]] = None,
                  dtype: torch.dtype = torch.bfloat16,
-                 layer_state: Optional[Sequence[dict]] = None):
+                 layer_state: Optional[Sequence[dict]] = None,
+                 model_state: Optional[dict] = None):
         self.layer_ids = list(layer_ids)
         self.local = {g: i for i, g in enumerate(self.layer_ids)}
         self.kv_bits = kv_bits
@@ -306,6 +307,11 @@ class KVCache:
                 {n: torch.zeros(batch, *shape, dtype=dt, device=device)
                  for n, (shape, dt) in (ls or {}).items()}
                 for ls in layer_state]
+        # per-slot state that belongs to no layer (the embedding's last
+        # token, ...): name -> tensor [B, ...], handled like the layers'
+        self.model_state: dict = {
+            n: torch.zeros(batch, *shape, dtype=dt, device=device)
+            for n, (shape, dt) in (model_state or {}).items()}
         if layer_dims is not None:
             # heterogeneous stacks: one (kv_heads, k_dim, v_dim) per local
             # layer -> per-layer tensors [B, Hkv_l, Smax, D_l] (self.k[li]
@@ -343,6 +349,7 @@ class KVCache:
         c.idle = self.idle[s:s + 1]
         c.state = [{n: t[s:s + 1] for n, t in st.items()}
                    for st in self.state]
+        c.model_state = {n: t[s:s + 1] for n, t in self.model_state.items()}
         if isinstance(self.k, list):
             c.k = [None if t is None else t[s:s + 1] for t in self.k]
             c.v = [None if t is None else t[s:s + 1] for t in self.v]
@@ -372,6 +379,8 @@ class KVCache:
                                              device=t.device)], dim=axis)
         self.state = [{n: pad(t, 0) for n, t in st.items()}
                       for st in self.state]
+        self.model_state = {n: pad(t, 0)
+                            for n, t in self.model_state.items()}
         self.idle = pad(self.idle, 0)
         if isinstance(self.k, list):
             self.k = [None if t is None else pad(t, 0) for t in self.k]

@@ -79,6 +79,13 @@ class ModelConfig:
     # hyper-connections (komizen): number of residual streams a layer mixes
     # (0 = one plain residual)
     hc_streams: int = 0
+    # hashed pair embedding (lurisun): {"buckets", "mul_prev", "mul_cur"} of
+    # the table added to the token embedding; None = no such table
+    pair_embedding: Optional[dict] = None
+    # taps of the causal convolution over a mixer's input (lurisun); 0 = none
+    input_conv_taps: int = 0
+    # factor on the output logits
+    logit_scale: float = 1.0
     # "bfloat16": bf16 weights/activations with 32-bit accumulation;
     # "float32": weights, activations and matrix products in true fp32
     # (honoured by the model families that implement it)
@@ -279,8 +286,75 @@ class ModelConfig:
         )
 
     @classmethod
+    def from_lurisun(cls, cfg: dict,
+                     quant: Optional[QuantConfig] = None) -> "ModelConfig":
+        """Lurisun checkpoints list their layers: {"architecture":
+        "Lurisun", "vocab", "width", "norm": {"eps"}, "canon": {"taps"}
+        (optional), "embedding": {"bigram": {"buckets", "mul_prev",
+        "mul_cur"}} (optional), "logit_scale" (optional), "layers":
+        [{"type": "lightning" | "attention" | "latent_attention", "mixer":
+        {...}, "mlp": {"kind": "dense", "ff"} | null}, ...]}. Every size is
+        per layer."""
+        need = {"lightning": ("decay", "dim", "heads", "vdim"),
+                "attention": ("dim", "heads", "kv_heads", "mask", "scale",
+                              "vdim"),
+                "latent_attention": ("dim", "heads", "kv_rank", "mask",
+                                     "q_rank", "scale", "vdim")}
+        specs = [dict(s) for s in cfg["layers"]]
+        for i, s in enumerate(specs):
+            kind, m = s.get("type"), s.get("mixer") or {}
+            if kind not in need:
+                raise ValueError(f"lurisun layer {i}: unknown mixer type "
+                                 f"{kind!r}")
+            missing = [k for k in need[kind] if k not in m]
+            if missing:
+                raise ValueError(f"lurisun layer {i}: mixer lacks {missing}")
+            if kind == "lightning" and len(m["decay"]) != m["heads"]:
+                raise ValueError(f"lurisun layer {i}: one decay per head")
+            if kind == "attention":
+                if m["heads"] % m["kv_heads"]:
+                    raise ValueError(f"lurisun layer {i}: heads % kv_heads")
+                if m["vdim"] != m["dim"]:
+                    raise ValueError(f"lurisun layer {i}: the values are "
+                                     "the key projections (vdim == dim)")
+                rot = m.get("rot")
+                if rot and (int(rot["dims"]) % 2
+                            or int(rot["dims"]) > m["dim"]):
+                    raise ValueError(f"lurisun layer {i}: rot.dims must be "
+                                     "even and at most dim")
+            if kind != "lightning" and int(m["mask"]["size"]) < 1:
+                raise ValueError(f"lurisun layer {i}: mask.size")
+            ff = s.get("mlp")
+            if ff is not None and ff.get("kind", "dense") != "dense":
+                raise ValueError(f"lurisun layer {i}: unknown feed-forward "
+                                 f"kind {ff.get('kind')!r}")
+        att = next((s["mixer"] for s in specs if s["type"] == "attention"),
+                   specs[0]["mixer"])
+        ffs = [s["mlp"]["ff"] for s in specs if s.get("mlp") is not None]
+        pair = (cfg.get("embedding") or {}).get("bigram")
+        return cls(
+            model_type="lurisun",
+            hidden_size=cfg["width"],
+            num_layers=len(specs),
+            num_q_heads=att["heads"],
+            num_kv_heads=att.get("kv_heads", 1),
+            head_dim=att["dim"],
+            v_head_dim=att["vdim"],
+            intermediate_size=max(ffs) if ffs else 0,
+            vocab_size=cfg["vocab"],
+            rms_eps=cfg["norm"]["eps"],
+            layer_specs=specs,
+            pair_embedding=dict(pair) if pair else None,
+            input_conv_taps=int((cfg.get("canon") or {}).get("taps") or 0),
+            logit_scale=float(cfg.get("logit_scale", 1.0)),
+            quant=quant,
+        )
+
+    @classmethod
     def from_hf(cls, cfg: dict, quant: Optional[QuantConfig] = None) -> "ModelConfig":
         arch = str(cfg.get("architecture", "")).lower()
+        if arch == "lurisun" or cfg.get("model_type") == "lurisun":
+            return cls.from_lurisun(cfg, quant)
         if arch == "posudra" or cfg.get("model_type") == "posudra":
             return cls.from_posudra(cfg, quant)
         if arch == "gegorax" or cfg.get("model_type") == "gegorax":
@@ -441,6 +515,53 @@ def komizen_config(width: int, vocab: int, pattern: str = "ldm",
     return cfg
 
 
+def lurisun_config(width: int, vocab: int, pattern: str = "nla",
+                   layers: int = 0, heads: int = 4, kv_heads: int = 2,
+                   dim: int = 32, rot_dims: int = 16, chunk: int = 24,
+                   latent_heads: int = 4, latent_dim: int = 16,
+                   latent_vdim: int = 24, kv_rank: int = 32, q_rank: int = 48,
+                   window: int = 20, lin_heads: int = 4, lin_dim: int = 16,
+                   lin_vdim: int = 32, decay: Optional[list] = None,
+                   ff: int = 192, taps: int = 4, buckets: int = 509,
+                   mul_prev: int = 53, mul_cur: int = 29,
+                   logit_scale: float = 1.0, rot_base: float = 10000.0,
+                   eps: float = 1e-6) -> dict:
+    """A lurisun stack in the checkpoint's config.json layout. ``pattern``
+    repeats over ``layers`` layers (default: once): 'n' = constant-decay
+    linear attention, 'a' = chunked sigmoid attention, 'l' = windowed latent
+    attention; every layer has a dense gated feed-forward when ``ff`` > 0.
+    ``taps`` 0: no input convolution; ``buckets`` 0: no pair table."""
+    if decay is None:
+        decay = [1.0 - 2.0 ** -(2 + 2 * h) for h in range(lin_heads)]
+    att = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim,
+           "scale": dim ** -0.5, "mask": {"size": chunk}}
+    if rot_dims:
+        att["rot"] = {"base": rot_base, "dims": rot_dims}
+    mix = {
+        "n": ("lightning", {"heads": lin_heads, "dim": lin_dim,
+                            "vdim": lin_vdim, "decay": list(decay)}),
+        "a": ("attention", att),
+        "l": ("latent_attention",
+              {"heads": latent_heads, "dim": latent_dim, "vdim": latent_vdim,
+               "kv_rank": kv_rank, "q_rank": q_rank,
+               "scale": latent_dim ** -0.5, "mask": {"size": window}}),
+    }
+    out = []
+    for i in range(layers or len(pattern)):
+        kind, m = mix[pattern[i % len(pattern)]]
+        out.append({"type": kind, "mixer": dict(m),
+                    "mlp": {"kind": "dense", "ff": ff} if ff else None})
+    cfg = {"architecture": "Lurisun", "vocab": vocab, "width": width,
+           "norm": {"eps": eps}, "logit_scale": logit_scale, "layers": out}
+    if taps:
+        cfg["canon"] = {"taps": taps}
+    if buckets:
+        cfg["embedding"] = {"bigram": {"buckets": buckets,
+                                       "mul_prev": mul_prev,
+                                       "mul_cur": mul_cur}}
+    return cfg
+
+
 # Known configs for synthetic benchmarking (random-init weights; no network).
 PRESETS: dict[str, dict] = {
     "llama-3-8b": dict(model_type="llama", hidden_size=4096, num_hidden_layers=32,
@@ -508,6 +629,8 @@ PRESETS: dict[str, dict] = {
                                    expert_ff=64, shared_ff=64, side_dim=16),
     "komizen-tiny": komizen_config(128, 256, "ldm", layers=4, loop=(1, 3, 2),
                                    embedding_scale=4.0),
+    "lurisun-tiny": lurisun_config(128, 256, "nla", layers=4,
+                                   logit_scale=0.5),
     "tiny": dict(model_type="llama", hidden_size=128, num_hidden_layers=4,
                  num_attention_heads=2, num_key_value_heads=2, head_dim=64,
                  intermediate_size=256, vocab_size=256, rope_theta=10000.0),

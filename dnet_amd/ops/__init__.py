@@ -351,7 +351,10 @@ def swiglu(gu: torch.Tensor) -> torch.Tensor:
     if gu.is_cuda:
         i = gu.shape[-1] // 2
         y = torch.empty(*gu.shape[:-1], i, dtype=gu.dtype, device=gu.device)
-        _native().swiglu(gu, y)
+        if gu.dtype == torch.bfloat16 and i % 8 == 0:
+            _native().swiglu(gu, y)
+        else:           # fp32 models, widths that are no multiple of 8
+            _native().silu_mul_halves(gu.contiguous(), y)
         return y
     return ref.swiglu(gu)
 
@@ -512,7 +515,8 @@ def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
              pos: torch.Tensor, T: int, scale: float, lens=None, slots=None,
              temp=None, softcap: float = 0.0, dist_r1=None, dist_r2=None,
              sinks=None, window: int = 0, pool_k=None, pool_v=None,
-             pool: int = 0, v_dim: int = 0) -> torch.Tensor:
+             pool: int = 0, v_dim: int = 0, chunk: int = 0,
+             sig_bias=None) -> torch.Tensor:
     """Causal attention against the cache with per-head temperature, tanh
     soft cap, logarithmic distance penalty and a sink in the softmax
     denominator (each optional). One entry point for decode (T=1) and
@@ -521,7 +525,12 @@ def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
     ``pool`` > 0 every whole block of ``pool`` positions before the window
     is seen as one entry of the pooled caches (see ``kv_pool_update``).
     ``vcache`` None (latent attention): the values are the first ``v_dim``
-    entries of the key rows, which the kernels then stage once for both."""
+    entries of the key rows, which the kernels then stage once for both.
+    ``chunk`` > 0: a query sees only the keys of its own block of ``chunk``
+    positions (blocks count from position 0). ``sig_bias`` fp32 [Hq]: no
+    softmax, the weight of a visible key is sigmoid(score + sig_bias[h])."""
+    if sig_bias is not None:
+        assert sinks is None and not pool
     if pool:
         assert window and pool_k is not None and pool_v is not None
     if vcache is None:
@@ -540,8 +549,11 @@ def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
             if window:
                 span = min(span, window + 64
                            + (pool_k.shape[2] if pool else 0))
+            if chunk:
+                span = min(span, chunk + 64)
             G = Hq // Hkv
             if (q.dtype == torch.bfloat16 and G >= 16 and not pool
+                    and not chunk and sig_bias is None
                     and D % 8 == 0 and Dv % 8 == 0):
                 # grouped heads on the matrix cores (the extension picks the
                 # kernel by the same rule): 64 heads per workgroup, splits of
@@ -564,11 +576,12 @@ def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
                            scale, temp, softcap or 0.0, dist_r1, dist_r2,
                            sinks, window or 0, partials, splits,
                            pool_k if pool else None,
-                           pool_v if pool else None, pool or 0, Dv)
+                           pool_v if pool else None, pool or 0, Dv,
+                           chunk or 0, sig_bias)
         return out
     return ref.attn_mod(q, kcache, vcache, pos, T, scale, lens, slots, temp,
                         softcap, dist_r1, dist_r2, sinks, window, pool_k,
-                        pool_v, pool, v_dim)
+                        pool_v, pool, v_dim, chunk, sig_bias)
 
 
 # ---- pooled-block caches, short convolutions, linear recurrences ----
@@ -778,3 +791,78 @@ def moe_weighted_sum(d, we) -> torch.Tensor:
         _native().moe_weighted_sum(d.contiguous(), we, out)
         return out
     return ref.moe_weighted_sum(d, we)
+
+
+# ---- hashed pair embedding, residual convolution, constant-decay linear
+# attention, sigmoid-weighted chunked attention (lurisun) ----
+# csrc/token_mix.hip.cpp, csrc/attn_mod.hip.cpp. Embedding sums, the
+# convolution over the fp32 residual, the recurrent state, norms and angles
+# are fp32 whatever the activation dtype.
+
+def pair_hash_embed(tokens, embed, table, prev, pos, buckets: int,
+                    mul_prev: int, mul_cur: int, lens=None,
+                    slots=None) -> torch.Tensor:
+    """embed[token] + table[hash(previous, token)] as fp32 [B, T, W]; the
+    slot's last token (``prev`` int32 [Bc]) is read for the first token of a
+    portion and advanced. See ``reference.pair_hash_embed``."""
+    if tokens.is_cuda:
+        B, T = tokens.shape
+        out = torch.empty(B, T, embed.shape[1], dtype=torch.float32,
+                          device=tokens.device)
+        _native().pair_hash_embed(tokens.contiguous(), embed, table, prev,
+                                  out, pos, lens, slots, buckets, mul_prev,
+                                  mul_cur)
+        return out
+    return ref.pair_hash_embed(tokens, embed, table, prev, pos, buckets,
+                               mul_prev, mul_cur, lens, slots)
+
+
+def causal_conv_residual(x, w, state, pos, T: int, out_dtype: torch.dtype,
+                         lens=None, slots=None) -> torch.Tensor:
+    """x + conv(x) over the fp32 rows x [B*T, C] (no bias, no activation);
+    ``state`` fp32 [Bc, taps-1, C] is each slot's input tail."""
+    if x.is_cuda:
+        y = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        _native().causal_conv_residual(x, w, state, y, pos, lens, slots, T)
+        return y
+    return ref.causal_conv_residual(x, w, state, pos, T, out_dtype, lens,
+                                    slots)
+
+
+def decay_scan(src, q0: int, k0: int, v0: int, decay, state, pos, T: int,
+               H: int, d: int, dv: int, lens=None, slots=None) -> torch.Tensor:
+    """Constant-decay linear attention over SiLU(q), SiLU(k), SiLU(v) taken
+    from columns of ``src``: S <- decay[h] S + k v^T, o = S^T q (fp32)."""
+    if src.is_cuda:
+        # padded rows of a ragged batch are never written by the kernel
+        o = (torch.zeros if lens is not None else torch.empty)(
+            src.shape[0], H * dv, dtype=torch.float32, device=src.device)
+        _native().decay_scan(src, q0, k0, v0, decay, state, o, pos, lens,
+                             slots, T, H, d, dv)
+        return o
+    return ref.decay_scan(src, q0, k0, v0, decay, state, pos, T, H, d, dv,
+                          lens, slots)
+
+
+def qknorm_half_append(qk, qw, kw, eps: float, nq: int, nkv: int, d: int,
+                       rot_freq, kcache, vcache, pos, T: int, lens=None,
+                       slots=None) -> torch.Tensor:
+    """Whole-projection RMS norm of q and k, half-split rotation (channel i
+    with i + n), keys appended to ``kcache`` and the raw key projections as
+    values to ``vcache``; returns the queries."""
+    if qk.is_cuda:
+        q = torch.empty(qk.shape[0], nq * d, dtype=qk.dtype, device=qk.device)
+        _native().qknorm_half_append(qk, qw, kw, q, kcache, vcache, pos, lens,
+                                     slots, eps, nq, nkv, d, T, rot_freq)
+        return q
+    return ref.qknorm_half_append(qk, qw, kw, eps, nq, nkv, d, rot_freq,
+                                  kcache, vcache, pos, T, lens, slots)
+
+
+def mul_sigmoid(a, gate_src, col0: int) -> torch.Tensor:
+    """a [M, N] * sigmoid(gate_src[:, col0:col0+N])."""
+    if a.is_cuda:
+        y = torch.empty_like(a)
+        _native().mul_sigmoid(a.contiguous(), gate_src, col0, y)
+        return y
+    return ref.mul_sigmoid(a, gate_src, col0)

@@ -17,6 +17,12 @@
 // (block means written by kv_pool_update) for every c < (i - window + 1) /
 // pool, in the same softmax and without a distance penalty.
 //
+// Chunked visibility (chunk > 0): a query sees key j only inside its own block
+// of `chunk` positions, j >= (i / chunk) * chunk, blocks counted from position
+// 0. Sigmoid weights (sbias given): no softmax; a visible key weighs
+// sigmoid(s_ij + sbias[h]) and the weights are not normalized over the keys
+// (rows and prefill kernels; no sink, no pooled entries).
+//
 // Three kernels:
 //  * attn_mod_rows<T>: flash-decode layout. One workgroup per (q tile, kv
 //    head, batch row): K/V chunks of 64 positions are staged through LDS once
@@ -104,7 +110,8 @@ struct ModParams {
   const float* sinks;
   const void* pk;      // pooled caches (same dtype as the cache) or null
   const void* pv;
-  int T, Bc, Hq, Hkv, Smax, D, DV, QT, window, pool, Sp;
+  const float* sbias;  // per-head bias of the sigmoid weights, or null
+  int T, Bc, Hq, Hkv, Smax, D, DV, QT, window, pool, Sp, chunk;
   // VS: elements between consecutive value rows of the cache. vshare: the
   // values are the first DV entries of the key rows (latent attention), the
   // value pointer is the key pointer and VS = D.
@@ -126,6 +133,10 @@ template <bool FAST> __device__ __forceinline__ float m_exp(float x) {
 template <bool FAST> __device__ __forceinline__ float m_tanh(float x) {
   return FAST ? 1.f - 2.f * __builtin_amdgcn_rcpf(__expf(2.f * x) + 1.f)
               : tanhf(x);
+}
+template <bool FAST> __device__ __forceinline__ float m_sigmoid(float x) {
+  return FAST ? __builtin_amdgcn_rcpf(1.f + __expf(-x))
+              : 1.f / (1.f + expf(-x));
 }
 template <bool FAST> __device__ __forceinline__ float m_log1p(float x) {
   return FAST ? __logf(1.f + x) : log1pf(x);
@@ -196,8 +207,9 @@ __global__ __launch_bounds__(256) void attn_mod_rows(
   }
 
   // per-wave query rows r = wid + 4*rr
-  float m[4], l[4], acc[4][4], tmp[4], r1[4], r2[4];
-  int qi[4];
+  float m[4], l[4], acc[4][4], tmp[4], r1[4], r2[4], sb[4];
+  int qi[4], cb[4];
+  const bool sig = P.sbias != nullptr;
 #pragma unroll
   for (int rr = 0; rr < 4; ++rr) {
     const int r = wid + 4 * rr;
@@ -207,7 +219,10 @@ __global__ __launch_bounds__(256) void attn_mod_rows(
     tmp[rr] = P.scale * (P.temp ? P.temp[h] : 1.f);
     r1[rr] = P.r1 ? P.r1[h] : 0.f;
     r2[rr] = P.r1 ? P.r2[h] : 0.f;
-    m[rr] = -1e30f;
+    sb[rr] = sig ? P.sbias[h] : 0.f;
+    // first position of the query's block (chunked visibility)
+    cb[rr] = (P.chunk > 0 && qi[rr] >= 0) ? (qi[rr] / P.chunk) * P.chunk : 0;
+    m[rr] = sig ? 0.f : -1e30f;
     l[rr] = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[rr][j] = 0.f;
@@ -215,8 +230,8 @@ __global__ __launch_bounds__(256) void attn_mod_rows(
   const float cap = P.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
 
   const int kv_end = min(p0 + t0 + nt, P.Smax);          // exclusive
-  const int kv_begin =
-      P.window > 0 ? max(0, p0 + t0 - P.window + 1) : 0;
+  int kv_begin = P.window > 0 ? max(0, p0 + t0 - P.window + 1) : 0;
+  if (P.chunk > 0) kv_begin = max(kv_begin, ((p0 + t0) / P.chunk) * P.chunk);
   const int64_t kbase = ((int64_t)slot * P.Hkv + hkv) * P.Smax * D;
   const int64_t vbase = ((int64_t)slot * P.Hkv + hkv) * P.Smax * P.VS;
   const int VS = P.VS;
@@ -275,16 +290,23 @@ __global__ __launch_bounds__(256) void attn_mod_rows(
       const int j = s0 + lane;
       bool live = lane < valid && j < lim;
       if (!pooled && P.window > 0) live = live && (j > i - P.window);
+      if (P.chunk > 0) live = live && (j >= cb[rr]);
       float s = dot_lds(&k_lds[lane * PK], &q_lds[r * PK], D) * tmp[rr];
       if (cap > 0.f) s = cap * m_tanh<FAST>(s * inv_cap);
       if (P.r1 && !pooled)
         s -= r1[rr] * m_log1p<FAST>(r2[rr] * (float)max(i - j, 0));
-      if (!live) s = -INFINITY;
-      const float mn = fmaxf(m[rr], wave_all_max(s));
-      const float alpha = m_exp<FAST>(m[rr] - mn);
-      const float p = live ? m_exp<FAST>(s - mn) : 0.f;
-      l[rr] = l[rr] * alpha + wave_all_sum(p);
-      m[rr] = mn;
+      float alpha, p;
+      if (sig) {                            // wave-uniform
+        alpha = 1.f;
+        p = live ? m_sigmoid<FAST>(s + sb[rr]) : 0.f;
+      } else {
+        if (!live) s = -INFINITY;
+        const float mn = fmaxf(m[rr], wave_all_max(s));
+        alpha = m_exp<FAST>(m[rr] - mn);
+        p = live ? m_exp<FAST>(s - mn) : 0.f;
+        l[rr] = l[rr] * alpha + wave_all_sum(p);
+        m[rr] = mn;
+      }
       p_lds[wid * kChunkR + lane] = p;
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // wave-local slab
       const int vis = min(valid, lim - s0);
@@ -359,7 +381,7 @@ __global__ __launch_bounds__(256) void attn_mod_rows(
       c = m_exp<FAST>(m[rr] - m2);
       l[rr] = l[rr] * c + m_exp<FAST>(sk - m2);
     }
-    const float inv = l[rr] > 0.f ? c / l[rr] : 0.f;
+    const float inv = sig ? 1.f : (l[rr] > 0.f ? c / l[rr] : 0.f);
     T* op = out + ((int64_t)b * P.T + t) * P.Hq * DV + (int64_t)h * DV;
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) {
@@ -380,9 +402,17 @@ __global__ __launch_bounds__(64) void attn_mod_combine(
     const float* __restrict__ partial, T* __restrict__ out,
     const float* __restrict__ sinks, const int* __restrict__ pos,
     const int* __restrict__ slots, const int Hq, const int DV,
-    const int splits, const int Bc) {
+    const int splits, const int Bc, const int plain_sum) {
   const int b = blockIdx.x / Hq, h = blockIdx.x % Hq;
   const float* pp = partial + (int64_t)blockIdx.x * splits * (DV + 2);
+  if (plain_sum) {             // unnormalized weights: the splits just add
+    for (int dv = threadIdx.x; dv < DV; dv += 64) {
+      float a = 0.f;
+      for (int s = 0; s < splits; ++s) a += pp[s * (DV + 2) + dv];
+      stv<T>(out + (int64_t)blockIdx.x * DV + dv, a);
+    }
+    return;
+  }
   float M = -1e30f;
   for (int s = 0; s < splits; ++s) M = fmaxf(M, pp[s * (DV + 2) + DV]);
   if (sinks) M = fmaxf(M, sinks[h]);
@@ -462,6 +492,8 @@ __global__ __launch_bounds__(256) void attn_mod_mfma(
   const float sc_t = P.scale * (P.temp ? P.temp[h] : 1.f);
   const float cap = P.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
   const float r1 = P.r1 ? P.r1[h] : 0.f, r2 = P.r1 ? P.r2[h] : 0.f;
+  const bool sig = P.sbias != nullptr;
+  const float sbias = sig ? P.sbias[h] : 0.f;
 
   const int q_hi = min(tile0 + 63, n - 1);
   const short* kp_tok = kp;
@@ -476,6 +508,8 @@ __global__ __launch_bounds__(256) void attn_mod_mfma(
   int s_begin = 0;
   if (!pooled && P.window > 0)
     s_begin = max(0, p0 + tile0 - P.window + 1) & ~(ST - 1);
+  if (!pooled && P.chunk > 0)
+    s_begin = max(s_begin, (((p0 + tile0) / P.chunk) * P.chunk) & ~(ST - 1));
   kp = pooled ? reinterpret_cast<const short*>(P.pk) +
                     ((int64_t)slot * P.Hkv + hk) * P.Sp * D
               : kp_tok;
@@ -531,10 +565,16 @@ __global__ __launch_bounds__(256) void attn_mod_mfma(
           if (P.r1) val -= r1 * __logf(1.f + r2 * (float)max(i - j, 0));
           dead = (j > i) || (qq >= n) || (j >= P.Smax);
           if (P.window > 0) dead |= (j <= i - P.window);
+          if (P.chunk > 0) dead |= (j < (i / P.chunk) * P.chunk);
         }
-        p_val[sub][r] = dead ? -INFINITY : val;
+        if (sig)
+          p_val[sub][r] =
+              dead ? 0.f : __builtin_amdgcn_rcpf(1.f + __expf(-(val + sbias)));
+        else
+          p_val[sub][r] = dead ? -INFINITY : val;
       }
     }
+    if (!sig)
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       float mx = fmaxf(p_val[0][r], p_val[1][r]);
@@ -586,7 +626,7 @@ __global__ __launch_bounds__(256) void attn_mod_mfma(
       c = __expf(m_run[r] - m2);
       l_run[r] = l_run[r] * c + __expf(sk - m2);
     }
-    const float inv = l_run[r] > 0.f ? c / l_run[r] : 0.f;
+    const float inv = sig ? 1.f : (l_run[r] > 0.f ? c / l_run[r] : 0.f);
     short* op = out + ((int64_t)b * P.T + qq) * P.Hq * DV + (int64_t)h * DV;
 #pragma unroll
     for (int nn = 0; nn < NV; ++nn) {
@@ -828,7 +868,8 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache,
               c10::optional<torch::Tensor> partials, int64_t splits,
               c10::optional<torch::Tensor> pool_k,
               c10::optional<torch::Tensor> pool_v, int64_t pool,
-              int64_t v_dim) {
+              int64_t v_dim, int64_t chunk,
+              c10::optional<torch::Tensor> sig_bias) {
   // no value cache: values = the first v_dim entries of the key rows
   const bool vshare = !vcache_opt.has_value();
   const torch::Tensor& vcache = vshare ? kcache : *vcache_opt;
@@ -865,6 +906,12 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache,
   P.r1 = opt_f32(dist_r1, Hq, "r1 fp32 [Hq]");
   P.r2 = opt_f32(dist_r2, Hq, "r2 fp32 [Hq]");
   P.sinks = opt_f32(sinks, Hq, "sinks fp32 [Hq]");
+  P.sbias = opt_f32(sig_bias, Hq, "sig_bias fp32 [Hq]");
+  P.chunk = (int)std::max<int64_t>(0, chunk);
+  const bool sig = P.sbias != nullptr;
+  DNET_CHECK(!sig || (!sinks.has_value() && pool == 0),
+             "sigmoid weights take no sink and no pooled entries");
+  DNET_CHECK(P.chunk == 0 || pool == 0, "chunks take no pooled entries");
   P.T = (int)T; P.Bc = Bc; P.Hq = Hq; P.Hkv = Hkv; P.Smax = Smax;
   P.D = D; P.DV = DV; P.window = (int)window;
   P.VS = vshare ? D : DV; P.vshare = vshare ? 1 : 0;
@@ -904,8 +951,8 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache,
   // bf16 decode with many heads per kv head: the grouped heads are the rows
   // of the matrix-core tile (the Python side sizes `partials` by the same
   // rule: attn_mod_heads_on_mfma)
-  if (!f32 && T == 1 && G >= kHeadsMfmaMinGroup && pool == 0 && D % 8 == 0 &&
-      DV % 8 == 0) {
+  if (!f32 && T == 1 && G >= kHeadsMfmaMinGroup && pool == 0 && !sig &&
+      P.chunk == 0 && D % 8 == 0 && DV % 8 == 0) {
     const int ns = (int)std::max<int64_t>(1, splits);
     DNET_CHECK(partials.has_value() &&
                    partials->scalar_type() == torch::kFloat32 &&
@@ -935,7 +982,7 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache,
 #undef AH
     hipLaunchKernelGGL((attn_mod_combine<short>), dim3((unsigned)(B * Hq)),
                        dim3(64), 0, stream, part, (short*)out.data_ptr(),
-                       P.sinks, P.pos, P.slots, Hq, DV, ns, Bc);
+                       P.sinks, P.pos, P.slots, Hq, DV, ns, Bc, 0);
     return;
   }
   // bf16 prompts: matrix-core kernel (head sizes padded to its tile classes)
@@ -990,7 +1037,8 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache,
     if (ns > 1)                                                             \
       hipLaunchKernelGGL((attn_mod_combine<TT>), dim3((unsigned)(B * Hq)),  \
                          dim3(64), 0, stream, part, (TT*)out.data_ptr(),    \
-                         P.sinks, P.pos, P.slots, Hq, DV, ns, Bc);          \
+                         P.sinks, P.pos, P.slots, Hq, DV, ns, Bc,           \
+                         sig ? 1 : 0);                                      \
   } while (0)
   if (f32) {
     if (vec) AR(float, true); else AR(float, false);

@@ -129,7 +129,33 @@ void attn_mod(torch::Tensor q, torch::Tensor kcache,
               c10::optional<torch::Tensor> partials, int64_t splits,
               c10::optional<torch::Tensor> pool_k,
               c10::optional<torch::Tensor> pool_v, int64_t pool,
-              int64_t v_dim);
+              int64_t v_dim, int64_t chunk,
+              c10::optional<torch::Tensor> sig_bias);
+void pair_hash_embed(torch::Tensor tokens, torch::Tensor embed,
+                     torch::Tensor table, torch::Tensor prev,
+                     torch::Tensor out, torch::Tensor pos,
+                     c10::optional<torch::Tensor> lens,
+                     c10::optional<torch::Tensor> slots, int64_t buckets,
+                     int64_t mul_prev, int64_t mul_cur);
+void causal_conv_residual(torch::Tensor x, torch::Tensor w, torch::Tensor state,
+                          torch::Tensor y, torch::Tensor pos,
+                          c10::optional<torch::Tensor> lens,
+                          c10::optional<torch::Tensor> slots, int64_t T);
+void decay_scan(torch::Tensor src, int64_t q0, int64_t k0, int64_t v0,
+                torch::Tensor decay, torch::Tensor state, torch::Tensor o,
+                torch::Tensor pos, c10::optional<torch::Tensor> lens,
+                c10::optional<torch::Tensor> slots, int64_t T, int64_t H,
+                int64_t d, int64_t dv);
+void qknorm_half_append(torch::Tensor qk, torch::Tensor qw, torch::Tensor kw,
+                        torch::Tensor qout, torch::Tensor kcache,
+                        torch::Tensor vcache, torch::Tensor pos,
+                        c10::optional<torch::Tensor> lens,
+                        c10::optional<torch::Tensor> slots, double eps,
+                        int64_t nq, int64_t nkv, int64_t d, int64_t T,
+                        c10::optional<torch::Tensor> rot_freq);
+void mul_sigmoid(torch::Tensor a, torch::Tensor gate_src, int64_t col0,
+                 torch::Tensor y);
+void silu_mul_halves(torch::Tensor gu, torch::Tensor y);
 void hc_write_read(torch::Tensor xs, c10::optional<torch::Tensor> y,
                    c10::optional<torch::Tensor> mix,
                    c10::optional<torch::Tensor> w_out,
@@ -239,6 +265,17 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("delta_scan", &dnet::delta_scan, "generalized delta-rule recurrence");
   m.def("hc_write_read", &dnet::hc_write_read,
         "residual streams: write a sublayer's result, read the next input");
+  m.def("pair_hash_embed", &dnet::pair_hash_embed,
+        "token embedding + hashed (previous, current) pair embedding");
+  m.def("causal_conv_residual", &dnet::causal_conv_residual,
+        "x + causal per-channel convolution of the fp32 residual");
+  m.def("decay_scan", &dnet::decay_scan,
+        "linear attention with a constant decay per head");
+  m.def("qknorm_half_append", &dnet::qknorm_half_append,
+        "whole-projection q/k norm, half-split rotation, cache append");
+  m.def("mul_sigmoid", &dnet::mul_sigmoid, "a * sigmoid(gate columns)");
+  m.def("silu_mul_halves", &dnet::silu_mul_halves,
+        "silu(gate half) * up half, any dtype and width");
   m.def("gated_delta_scan", &dnet::gated_delta_scan,
         "gated delta-rule recurrence");
   m.def("latent_append", &dnet::latent_append,

@@ -586,7 +586,8 @@ def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
              pos: torch.Tensor, T: int, scale: float, lens=None, slots=None,
              temp=None, softcap: float = 0.0, dist_r1=None, dist_r2=None,
              sinks=None, window: int = 0, pool_k=None, pool_v=None,
-             pool: int = 0, v_dim: int = 0) -> torch.Tensor:
+             pool: int = 0, v_dim: int = 0, chunk: int = 0,
+             sig_bias=None) -> torch.Tensor:
     """Causal attention against the cache with score modifiers, all in
     fp32: s = q.k * scale * temp[h]; s = cap*tanh(s/cap);
     s -= r1[h] * ln(1 + r2[h] * (i-j)); softmax whose denominator also
@@ -600,7 +601,12 @@ def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
     no distance penalty.
 
     ``vcache`` None: the values are the first ``v_dim`` entries of the key
-    rows (latent attention: one cached latent is key and value)."""
+    rows (latent attention: one cached latent is key and value).
+
+    ``chunk`` > 0: query i sees key j only inside its own block of ``chunk``
+    positions (j >= (i // chunk) * chunk; blocks count from position 0).
+    ``sig_bias`` fp32 [Hq]: no softmax; the weight of a visible key is
+    sigmoid(s + sig_bias[h]), not normalized over the keys."""
     Hkv, D = kcache.shape[1], kcache.shape[3]
     if vcache is None:
         vcache = kcache[..., :v_dim]
@@ -635,6 +641,16 @@ def attn_mod(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
         dead = dist < 0
         if window and window > 0:
             dead = dead | (dist >= window)
+        if chunk and chunk > 0:
+            dead = dead | (j < torch.div(i, chunk, rounding_mode="floor")
+                           * chunk)
+        if sig_bias is not None:
+            assert not pool and sinks is None
+            pr = torch.sigmoid(sc + sig_bias.float().view(Hkv, G, 1, 1))
+            pr = pr.masked_fill(dead, 0.0)
+            o = torch.einsum("hgts,hsd->thgd", pr, vv)
+            out[b * T:b * T + n] = o.reshape(n, Hq * Dv).to(q.dtype)
+            continue
         sc = sc.masked_fill(dead, float("-inf"))
         nb = 0
         if pool and window and window > 0:
@@ -1047,3 +1063,154 @@ def moe_route(logits: torch.Tensor, top: int, scale: float) -> torch.Tensor:
 def moe_weighted_sum(d: torch.Tensor, we: torch.Tensor) -> torch.Tensor:
     """d [E, T, W], we [T, E] -> fp32 [T, W] = sum_e we[t, e] d[e, t]."""
     return torch.einsum("te,etw->tw", we.float(), d.float())
+
+
+# ---- hashed pair embedding, residual convolution, constant-decay linear
+# attention, gated outputs (lurisun) ----
+
+def pair_hash_embed(tokens: torch.Tensor, embed: torch.Tensor,
+                    table: torch.Tensor, prev: torch.Tensor,
+                    pos: torch.Tensor, buckets: int, mul_prev: int,
+                    mul_cur: int, lens=None, slots=None) -> torch.Tensor:
+    """Token embedding plus a hashed embedding of the (previous, current)
+    token pair, fp32 [B, T, W]. tokens [B, T]; token (b,t) sits at position
+    pos[b]+t of slot slots[b]. Row of ``table`` [buckets+1, W]:
+    (previous * mul_prev + current * mul_cur) mod buckets, and row ``buckets``
+    at position 0. ``prev`` int32 [Bc] holds every slot's last token and is
+    advanced by the rows' real tokens (t < lens[b])."""
+    B, T = tokens.shape
+    out = embed[tokens.long()].float()
+    p, ln, sl = _row_index(B, T, pos, lens, slots, tokens.device)
+    for b in range(B):
+        n = int(min(ln[b], T))
+        if n <= 0:
+            continue
+        p0, s = int(p[b]), int(sl[b])
+        last = int(prev[s])
+        for t in range(n):
+            cur = int(tokens[b, t])
+            row = buckets if p0 + t == 0 else \
+                (last * mul_prev + cur * mul_cur) % buckets
+            out[b, t] += table[row].float()
+            last = cur
+        prev[s] = last
+    return out
+
+
+def causal_conv_residual(x: torch.Tensor, w: torch.Tensor,
+                         state: torch.Tensor, pos: torch.Tensor, T: int,
+                         out_dtype: torch.dtype, lens=None,
+                         slots=None) -> torch.Tensor:
+    """y = x + conv(x): per-channel causal convolution of the fp32 rows
+    x [B*T, C] without bias or activation, added to its input. w fp32
+    [C, taps] (last tap = current token); ``state`` fp32 [Bc, taps-1, C]
+    holds each slot's last taps-1 inputs (positions < 0 count as zero) and is
+    advanced. Returns [B*T, C] in ``out_dtype`` (padding rows zero)."""
+    C, taps = w.shape
+    M = x.shape[0]
+    B = M // T
+    out = torch.zeros(M, C, dtype=torch.float32, device=x.device)
+    p, ln, sl = _row_index(B, T, pos, lens, slots, x.device)
+    wf = w.float()
+    for b in range(B):
+        n = int(min(ln[b], T))
+        if n <= 0:
+            continue
+        p0, s = int(p[b]), int(sl[b])
+        hist = state[s].float().clone()
+        for j in range(taps - 1):
+            if p0 - (taps - 1) + j < 0:
+                hist[j] = 0.0
+        seq = torch.cat([hist, x[b * T:b * T + n].float()])
+        acc = x[b * T:b * T + n].float().clone()
+        for j in range(taps):
+            acc = acc + seq[j:j + n] * wf[:, j]
+        out[b * T:b * T + n] = acc
+        if taps > 1:
+            state[s] = seq[n:].to(state.dtype)
+    return out.to(out_dtype)
+
+
+def decay_scan(src: torch.Tensor, q0: int, k0: int, v0: int,
+               decay: torch.Tensor, state: torch.Tensor, pos: torch.Tensor,
+               T: int, H: int, d: int, dv: int, lens=None,
+               slots=None) -> torch.Tensor:
+    """Linear attention with one constant decay per head, fp32. q, k [H*d]
+    and v [H*dv] are columns q0 / k0 / v0 of src [B*T, ld] with SiLU applied
+    here; per head S <- decay[h] S + k v^T (S [d, dv]), o = S^T q. ``state``
+    fp32 [Bc, H, d, dv] per slot: zero at position 0, advanced by the rows'
+    real tokens. Returns fp32 [B*T, H*dv] (padding rows zero)."""
+    M = src.shape[0]
+    B = M // T
+    out = torch.zeros(M, H * dv, dtype=torch.float32, device=src.device)
+    p, ln, sl = _row_index(B, T, pos, lens, slots, src.device)
+    f = src.float()
+    act = torch.nn.functional.silu
+    g = decay.float().view(H, 1, 1)
+    for b in range(B):
+        n = int(min(ln[b], T))
+        if n <= 0:
+            continue
+        p0, s = int(p[b]), int(sl[b])
+        rows = f[b * T:b * T + n]
+        q = act(rows[:, q0:q0 + H * d]).view(n, H, d)
+        k = act(rows[:, k0:k0 + H * d]).view(n, H, d)
+        v = act(rows[:, v0:v0 + H * dv]).view(n, H, dv)
+        S = state[s].float().clone() if p0 > 0 else \
+            torch.zeros(H, d, dv, dtype=torch.float32, device=src.device)
+        for t in range(n):
+            S = g * S + k[t].unsqueeze(-1) * v[t].unsqueeze(-2)
+            out[b * T + t] = torch.einsum("hdv,hd->hv", S, q[t]).reshape(-1)
+        state[s] = S
+    return out
+
+
+def qknorm_half_append(qk: torch.Tensor, qw: torch.Tensor, kw: torch.Tensor,
+                       eps: float, nq: int, nkv: int, d: int,
+                       rot_freq: torch.Tensor | None, kcache: torch.Tensor,
+                       vcache: torch.Tensor, pos: torch.Tensor, T: int,
+                       lens=None, slots=None) -> torch.Tensor:
+    """qk [B*T, nq*d + nkv*d] = [q | k]. The cached VALUES are the key
+    projections as they come; the cached keys and the returned queries are
+    RMS-normalized over the whole projection (weights qw [nq*d], kw [nkv*d])
+    and then, per head, channel i < n pairs with channel i + n
+    (n = len(rot_freq)) and the pair turns by position * rot_freq[i]; the
+    channels from 2n on pass through. Statistics and angles fp32."""
+    M = qk.shape[0]
+    B = M // T
+    q, k = qk[:, :nq * d], qk[:, nq * d:]
+    qf = rmsnorm_rows(q, qw, eps, torch.float32).view(M, nq, d)
+    kf = rmsnorm_rows(k, kw, eps, torch.float32).view(M, nkv, d)
+    p, ln, sl = _row_index(B, T, pos, lens, slots, qk.device)
+    n = 0 if rot_freq is None else rot_freq.numel()
+    if n:
+        tpos = (p.view(B, 1) + torch.arange(T, device=qk.device)
+                ).reshape(M).to(torch.float32)
+        ang = tpos.view(M, 1) * rot_freq.float().view(1, -1)
+        c, s = torch.cos(ang).unsqueeze(1), torch.sin(ang).unsqueeze(1)
+
+        def turn(x):
+            out = x.clone()
+            u, v = x[..., :n], x[..., n:2 * n]
+            out[..., :n] = u * c - v * s
+            out[..., n:2 * n] = v * c + u * s
+            return out
+        qf, kf = turn(qf), turn(kf)
+    for b in range(B):
+        cnt = int(min(ln[b], T))
+        if cnt <= 0:
+            continue
+        p0, s_ = int(p[b]), int(sl[b])
+        kcache[s_, :, p0:p0 + cnt] = kf[b * T:b * T + cnt].transpose(0, 1) \
+            .to(kcache.dtype)
+        vcache[s_, :, p0:p0 + cnt] = k[b * T:b * T + cnt].reshape(
+            cnt, nkv, d).transpose(0, 1).to(vcache.dtype)
+    return qf.reshape(M, nq * d).to(qk.dtype)
+
+
+def mul_sigmoid(a: torch.Tensor, gate_src: torch.Tensor,
+                col0: int) -> torch.Tensor:
+    """a [M, N] * sigmoid(gate_src[:, col0:col0+N]), fp32 math."""
+    N = a.shape[1]
+    return (a.float() * torch.sigmoid(gate_src[:, col0:col0 + N].float())
+            ).to(a.dtype)

@@ -229,9 +229,23 @@ class RingExecutor:
 
     # ------------- one-rank step bodies (graph-capturable) -------------
 
+    def embed(self, tokens: torch.Tensor, kv, pos, lens=None, slots=None):
+        """The model's embedding of ``tokens`` ([B] decode step or [B, T]
+        prompt portion). Families whose embedding keeps per-slot state (the
+        previous token of a sequence) also get the cache and the rows'
+        geometry: first positions ``pos`` (int or int32 [B]), real lengths
+        and slots as for ``prefill_window``."""
+        if getattr(self.model, "embed_reads_cache", False):
+            return self.model.embed_tokens(tokens, kv=kv, pos=pos, lens=lens,
+                                           slots=slots)
+        return self.model.embed_tokens(tokens)
+
     def _decode_body(self, mb: int, r: int = 0):
         if self.is_first and r == 0:
-            self.hbuf[mb].copy_(self.model.embed_tokens(self.tokbuf[mb]))
+            kv = self.kvs[mb]
+            self.hbuf[mb].copy_(self.embed(
+                self.tokbuf[mb], kv, kv.pos,
+                lens=(~kv.idle).to(torch.int32)))
         elif self._needs_tokens:
             self.model.set_tokens(self.tokbuf[mb])
         if self.windows[r]:
@@ -336,8 +350,8 @@ class RingExecutor:
                 h = None
                 for r in range(self.rounds):
                     if self.is_first and r == 0:
-                        h = self.model.embed_tokens(
-                            tokens[mb, :, p0:p1].to(self.device)).clone()
+                        h = self.embed(tokens[mb, :, p0:p1].to(self.device),
+                                       self.kvs[mb], p0).clone()
                     else:
                         if h is None:
                             h = torch.empty(B, p1 - p0, H,
@@ -540,8 +554,16 @@ class RingExecutor:
                 h = None
                 for r in range(self.rounds):
                     if self.is_first and r == 0:
-                        h = self.model.embed_tokens(
-                            tok[:, p0:p1].to(self.device)).clone()
+                        if self.model.ragged_prefill:
+                            h = self.embed(
+                                tok[:, p0:p1].to(self.device), kv,
+                                start_t + p0,
+                                lens=(len_t - p0).clamp_(0, p1 - p0),
+                                slots=slot_t).clone()
+                        else:
+                            h = self.embed(tok[:, p0:p1].to(self.device),
+                                           kvslot,
+                                           start[grp[0]] + p0).clone()
                     else:
                         if h is None:
                             h = torch.empty(B, p1 - p0, H,

@@ -780,8 +780,8 @@ class ShardRuntime:
         p0 = st["p0"]
         p1 = min(p0 + chunk, T)
         kvslot = ex.kvs[0].slot(si)
-        h = ex.model.embed_tokens(
-            toks.view(1, T)[:, p0:p1].to(ex.device)).clone()
+        h = ex.embed(toks.view(1, T)[:, p0:p1].to(ex.device), kvslot,
+                     p0).clone()
         ex.model.prefill_window(h, ex.my_layers, kvslot, p0)
         st["p0"] = p1
         if p1 < T:

@@ -80,8 +80,8 @@ def get_model_metadata(model_dir: str) -> ModelMetadata:
             m = _LAYER_RE.match(ti.name)
             if m:
                 meta.layers.setdefault(int(m.group(1)), []).append(ti.name)
-            elif "embed_tokens" in ti.name or ti.name in ("embed",
-                                                          "side.embed"):
+            elif "embed_tokens" in ti.name or ti.name in (
+                    "embed", "side.embed", "bigram"):
                 meta.embed.append(ti.name)
             elif "lm_head" in ti.name or ti.name == "head":
                 meta.lm_head.append(ti.name)
