@@ -186,3 +186,64 @@ def forward(tokens, sd, cfg, dtype=torch.float32, layers_out=None):
             layers_out.append(x.clone())
     y = norm_plain(x, sd["final.norm"], eps)
     return (y @ sd["head"].T) * float(cfg.get("logit_scale", 1.0))
+
+
+def make_checkpoint(cfg, seed=0, dtype=torch.bfloat16, ff_gain=1.0):
+    """Random tensors for a config.json dict, under the checkpoint's names;
+    values are rounded to ``dtype`` (so a bfloat16 and a float32 run read the
+    same numbers)."""
+    g = torch.Generator().manual_seed(seed)
+    W, V = cfg["width"], cfg["vocab"]
+
+    def rn(*shape, std=1.0):
+        return (torch.randn(*shape, generator=g) * std).to(dtype)
+
+    def lin(out, inp, gain=1.0):
+        return rn(out, inp, std=gain * inp ** -0.5)
+
+    sd = {"embed": rn(V, W), "final.norm": 1 + rn(W, std=0.1),
+          "head": lin(V, W)}
+    bg = (cfg.get("embedding") or {}).get("bigram")
+    if bg:
+        sd["bigram"] = rn(int(bg["buckets"]) + 1, W, std=0.7)
+    taps = int((cfg.get("canon") or {}).get("taps") or 0)
+    for i, spec in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", spec["mixer"]
+        sd[p + "norm1"] = 1 + rn(W, std=0.1)
+        if taps:
+            sd[p + "canon1"] = rn(W, taps, std=0.4)
+        if spec["type"] == "lightning":
+            H, d, dv = m["heads"], m["dim"], m["vdim"]
+            sd.update({p + "mix.q": lin(H * d, W), p + "mix.k": lin(H * d, W),
+                       p + "mix.v": lin(H * dv, W),
+                       p + "mix.g": lin(H * dv, W),
+                       p + "mix.norm": 1 + rn(H * dv, std=0.1),
+                       p + "mix.o": lin(W, H * dv)})
+        elif spec["type"] == "attention":
+            H, G, d = m["heads"], m["kv_heads"], m["dim"]
+            sd.update({p + "mix.q": lin(H * d, W), p + "mix.k": lin(G * d, W),
+                       p + "mix.q.b": rn(H * d, std=0.2),
+                       p + "mix.k.b": rn(G * d, std=0.2),
+                       p + "mix.q.norm": 1 + rn(H * d, std=0.1),
+                       p + "mix.k.norm": 1 + rn(G * d, std=0.1),
+                       p + "mix.pb": rn(H, std=0.5) - 1.5,
+                       p + "mix.o": lin(W, H * m["vdim"])})
+        else:
+            H, d, dv = m["heads"], m["dim"], m["vdim"]
+            R, QR = m["kv_rank"], m["q_rank"]
+            sd.update({p + "mix.dq": lin(QR, W),
+                       p + "mix.dq.norm": 1 + rn(QR, std=0.1),
+                       p + "mix.uq": lin(H * d, QR, 2.0),
+                       p + "mix.dkv": lin(R, W),
+                       p + "mix.dkv.norm": 1 + rn(R, std=0.1),
+                       p + "mix.uk": lin(H * d, R, 2.0),
+                       p + "mix.uv": lin(H * dv, R),
+                       p + "mix.g": lin(H * dv, W),
+                       p + "mix.o": lin(W, H * dv)})
+        ff = spec.get("mlp")
+        if ff is not None:
+            sd.update({p + "norm2": (1 + rn(W, std=0.1)) * ff_gain,
+                       p + "mlp.gate": lin(ff["ff"], W),
+                       p + "mlp.up": lin(ff["ff"], W),
+                       p + "mlp.down": lin(W, ff["ff"])})
+    return sd
