@@ -56,7 +56,22 @@ _COMPARE_SIZES = [("2k", 2048, 16, 4, 128, 8192),
 def _family_hf(fam, W, H, KV, D, FF, layers, vocab, args):
     """config.json-style description of ``fam`` at the given layer sizes."""
     from dnet_amd.models.config import (gegorax_config, komizen_config,
-                                        posudra_config)
+                                        lurisun_config, posudra_config)
+    if fam == "lurisun":
+        # constant-decay linear attention, windowed latent attention and
+        # chunked sigmoid attention in turn; linear-attention heads of D x D
+        # state over the model width, 256 cached latent entries per token,
+        # window and chunk half the prompt, a 4-tap input convolution in
+        # every layer, a hashed pair table beside the embedding, dense gated
+        # feed-forwards
+        return lurisun_config(
+            W, vocab, "nla", layers=layers, heads=H, kv_heads=KV, dim=D,
+            rot_dims=D // 2, chunk=max(64, args.prompt_len // 2),
+            latent_heads=H, latent_dim=D, latent_vdim=D, kv_rank=256,
+            q_rank=max(256, W // 4), window=max(64, args.prompt_len // 2),
+            lin_heads=W // D, lin_dim=D, lin_vdim=D,
+            decay=[1.0 - 2.0 ** -(3 + h % 8) for h in range(W // D)], ff=FF,
+            taps=4, buckets=100003)
     if fam == "komizen":
         # latent attention (every second layer) with gated delta-rule and
         # mamba2 layers between; 192 + 64 cached entries per token; 4
@@ -97,7 +112,7 @@ def _family_hf(fam, W, H, KV, D, FF, layers, vocab, args):
 
 # family -> the closest existing family it is measured beside
 _COMPARE_WITH = {"posudra": "qwen3", "gegorax": "posudra",
-                 "komizen": "gegorax"}
+                 "komizen": "gegorax", "lurisun": "gegorax"}
 
 
 def compare_family(args, device):
@@ -105,7 +120,9 @@ def compare_family(args, device):
     one (posudra: qwen3 — dense, grouped heads, q/k norm; gegorax: posudra —
     one norm feeding parallel branches, fp32 residual, per-layer sizes;
     komizen: gegorax — attention beside state-space and delta-rule layers on
-    an fp32 residual with per-slot recurrent state) at
+    an fp32 residual with per-slot recurrent state; lurisun: gegorax —
+    windowed attention beside linear recurrences with per-slot state, dense
+    feed-forwards, fp32 residual) at
     equal layer sizes, bf16, random weights. One JSON line; the default
     workload is untouched."""
     new, old = args.compare_family, _COMPARE_WITH[args.compare_family]
@@ -194,7 +211,7 @@ def main():
                     help="GPU-resident layers per rank (0=all; <local layers "
                          "enables host-DRAM weight streaming)")
     ap.add_argument("--compare-family", default="",
-                    choices=["", "posudra", "gegorax", "komizen"],
+                    choices=["", "posudra", "gegorax", "komizen", "lurisun"],
                     help="instead of the default workload: throughput of "
                          "this family beside its closest existing one at "
                          "equal layer sizes")

@@ -81,7 +81,18 @@ bool is_f32(const torch::Tensor& t) { return t.scalar_type() == torch::kFloat32;
 // ---- hashed pair embedding ---------------------------------------------------
 // grid (B*T), one workgroup per token. Padding rows get the plain embedding
 // (their output is never used).
-template <typename T>
+template <typename T> __device__ __forceinline__ void ld4(const T* p, float (&v)[4]);
+template <> __device__ __forceinline__ void ld4<float>(const float* p, float (&v)[4]) {
+  const float4 q = *reinterpret_cast<const float4*>(p);
+  v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+}
+template <> __device__ __forceinline__ void ld4<short>(const short* p, float (&v)[4]) {
+  const short4v q = *reinterpret_cast<const short4v*>(p);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) v[e] = bits2f(q.x[e]);
+}
+
+template <typename T, bool V4>
 __global__ __launch_bounds__(256) void pair_hash_embed_kernel(
     const int64_t* __restrict__ tokens, const T* __restrict__ embed,
     const T* __restrict__ table, const int* __restrict__ prev,
@@ -106,10 +117,20 @@ __global__ __launch_bounds__(256) void pair_hash_embed_kernel(
   const T* er = embed + tok * W;
   const T* tr = pr >= 0 ? table + pr * W : nullptr;
   float* orow = out + row * W;
-  for (int i = threadIdx.x; i < W; i += blockDim.x) {
-    float v = ldx<T>(er + i);
-    if (tr) v += ldx<T>(tr + i);
-    orow[i] = v;
+  if constexpr (V4) {          // W % 4 == 0: 8 B / 16 B loads, 16 B stores
+    for (int i = threadIdx.x * 4; i < W; i += blockDim.x * 4) {
+      float v[4], u[4] = {0.f, 0.f, 0.f, 0.f};
+      ld4<T>(er + i, v);
+      if (tr) ld4<T>(tr + i, u);
+      *reinterpret_cast<float4*>(orow + i) =
+          make_float4(v[0] + u[0], v[1] + u[1], v[2] + u[2], v[3] + u[3]);
+    }
+  } else {
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+      float v = ldx<T>(er + i);
+      if (tr) v += ldx<T>(tr + i);
+      orow[i] = v;
+    }
   }
 }
 
@@ -426,14 +447,16 @@ void pair_hash_embed(torch::Tensor tokens, torch::Tensor embed,
   if (B * T == 0) return;
   const Rows g = make_rows(pos, lens, slots, B, T, prev.size(0));
   auto st = current_stream();
-#define PE(TT)                                                                 \
-  hipLaunchKernelGGL((pair_hash_embed_kernel<TT>), dim3((unsigned)(B * T)),    \
-                     dim3(256), 0, st, tokens.data_ptr<int64_t>(),             \
-                     (const TT*)embed.data_ptr(), (const TT*)table.data_ptr(), \
-                     prev.data_ptr<int>(), out.data_ptr<float>(), g, W,        \
-                     (int)embed.size(0), (int)buckets, mul_prev, mul_cur)
-  if (is_bf16(embed)) PE(short);
-  else if (is_f32(embed)) PE(float);
+#define PE(TT, VV)                                                             \
+  hipLaunchKernelGGL((pair_hash_embed_kernel<TT, VV>),                         \
+                     dim3((unsigned)(B * T)), dim3(256), 0, st,                \
+                     tokens.data_ptr<int64_t>(), (const TT*)embed.data_ptr(),  \
+                     (const TT*)table.data_ptr(), prev.data_ptr<int>(),        \
+                     out.data_ptr<float>(), g, W, (int)embed.size(0),          \
+                     (int)buckets, mul_prev, mul_cur)
+  const bool v4 = W % 4 == 0;
+  if (is_bf16(embed)) { if (v4) PE(short, true); else PE(short, false); }
+  else if (is_f32(embed)) { if (v4) PE(float, true); else PE(float, false); }
   else DNET_CHECK(false, "pair_hash_embed: dtype");
 #undef PE
   hipLaunchKernelGGL(pair_hash_state_kernel, dim3((unsigned)((B + 63) / 64)),

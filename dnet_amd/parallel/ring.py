@@ -242,10 +242,15 @@ class RingExecutor:
 
     def _decode_body(self, mb: int, r: int = 0):
         if self.is_first and r == 0:
-            kv = self.kvs[mb]
-            self.hbuf[mb].copy_(self.embed(
-                self.tokbuf[mb], kv, kv.pos,
-                lens=(~kv.idle).to(torch.int32)))
+            if getattr(self.model, "embed_reads_cache", False):
+                # idle rows neither read nor advance their slot's state
+                kv = self.kvs[mb]
+                self.hbuf[mb].copy_(self.embed(
+                    self.tokbuf[mb], kv, kv.pos,
+                    lens=(~kv.idle).to(torch.int32)))
+            else:
+                self.hbuf[mb].copy_(
+                    self.model.embed_tokens(self.tokbuf[mb]))
         elif self._needs_tokens:
             self.model.set_tokens(self.tokbuf[mb])
         if self.windows[r]:
