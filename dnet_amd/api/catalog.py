@@ -46,6 +46,8 @@ model_catalog: list[CatalogEntry] = [
                  tokenizer="byte", ci_test=True),
     CatalogEntry("komizen-tiny-random", preset="komizen-tiny",
                  tokenizer="byte", ci_test=True),
+    CatalogEntry("lurisun-tiny-random", preset="lurisun-tiny",
+                 tokenizer="byte", ci_test=True),
     CatalogEntry("openai/gpt-oss-20b", repo="openai/gpt-oss-20b"),
     CatalogEntry("deepseek-ai/DeepSeek-V2-Lite", repo="deepseek-ai/DeepSeek-V2-Lite"),
     # real checkpoints (local safetensors dir or pre-downloaded HF cache)

@@ -224,3 +224,36 @@ def test_looped_multi_stream_family_over_two_shards(cluster):
         assert texts[0] == texts[1]
         r = c.post(f"{api}/v1/unload_model")
         assert r.status_code == 200
+
+
+@pytest.mark.timeout(300)
+def test_embedding_state_family_over_two_shards(cluster):
+    """A family whose embedding keeps the sequence's last token and whose
+    layers keep convolution tails, recurrent states and caches of three kinds
+    (lurisun) split over the two shards: chats complete and repeat, also when
+    the slot is used again."""
+    api = cluster["api"]
+    name = "lurisun-tiny-random"
+    with httpx.Client(timeout=180) as c:
+        r = c.post(f"{api}/v1/prepare_topology_manual", json={
+            "model": name,
+            "assignments": [
+                {"instance": "shard0", "layers": [0, 1]},
+                {"instance": "shard1", "layers": [2, 3]}]})
+        assert r.status_code == 200, r.text
+        r = c.post(f"{api}/v1/load_model",
+                   json={"model": name, "max_tokens": 8})
+        assert r.status_code == 200, r.text
+        texts = []
+        for _ in range(2):          # greedy: the same prompt repeats exactly
+            r = c.post(f"{api}/v1/chat/completions", json={
+                "model": name, "stream": False, "max_tokens": 8,
+                "temperature": 0.0,
+                "messages": [{"role": "user", "content": "pairs please"}]})
+            assert r.status_code == 200, r.text
+            body = r.json()
+            assert body["usage"]["completion_tokens"] >= 1
+            texts.append(body["choices"][0]["message"]["content"])
+        assert texts[0] == texts[1]
+        r = c.post(f"{api}/v1/unload_model")
+        assert r.status_code == 200
