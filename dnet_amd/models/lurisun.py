@@ -112,14 +112,14 @@ class LurisunRingModel(RingModel):
 
     def make_kv_cache(self, batch: int, smax: int) -> KVCache:
         W = self.cfg.hidden_size
-        taps = max(int(self.cfg.input_conv_taps) - 1, 0)
+        conv = int(self.cfg.input_conv_taps)
         dims, states = [], []
         for lid in self.layer_ids:
             s = self._spec(lid)
             m = s["mixer"]
             st = {}
-            if taps:
-                st["conv"] = ((taps, W), torch.float32)
+            if conv:                # a one-tap convolution has an empty tail
+                st["conv"] = ((conv - 1, W), torch.float32)
             if s["type"] == "attention":
                 dims.append((m["kv_heads"], m["dim"], m["vdim"]))
             elif s["type"] == "latent_attention":

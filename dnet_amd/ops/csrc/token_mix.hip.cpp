@@ -150,7 +150,7 @@ __global__ void pair_hash_state_kernel(const int64_t* __restrict__ tokens,
 // grid (channel tiles, B * token tiles): a thread walks kTile consecutive
 // tokens of one channel with the sliding window of inputs in registers.
 constexpr int kTile = 16;
-constexpr int kMaxTaps = 8;
+constexpr int kMaxTaps = 16;
 
 template <typename TO>
 __global__ __launch_bounds__(256) void conv_residual_kernel(
@@ -472,7 +472,7 @@ void causal_conv_residual(torch::Tensor x, torch::Tensor w, torch::Tensor state,
   DNET_CHECK(w.dim() == 2 && is_f32(w) && w.is_contiguous() &&
                  w.size(0) == x.size(1), "w fp32 [C, taps]");
   const int C = w.size(0), taps = w.size(1);
-  DNET_CHECK(taps >= 1 && taps <= kMaxTaps, "1 <= taps <= 8");
+  DNET_CHECK(taps >= 1 && taps <= kMaxTaps, "1 <= taps <= 16");
   const int64_t M = x.size(0);
   DNET_CHECK(T > 0 && M % T == 0, "rows = B*T");
   const int64_t B = M / T;

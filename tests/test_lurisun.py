@@ -439,6 +439,12 @@ OTHER = [
     dict(pattern="nnal", layers=4, taps=6, heads=8, kv_heads=1, dim=8,
          rot_dims=4, chunk=1, window=1, lin_heads=2, lin_dim=4, lin_vdim=20,
          decay=[0.99, 0.3], mul_prev=1, mul_cur=1, buckets=1000),
+    # a one-tap convolution (no tail), odd width-independent sizes, sixteen
+    # query heads on one latent (the grouped-heads decode kernel in bf16)
+    dict(pattern="lna", layers=3, taps=1, latent_heads=16, latent_dim=6,
+         latent_vdim=5, kv_rank=24, q_rank=11, window=7, heads=3, kv_heads=3,
+         dim=14, rot_dims=6, chunk=13, lin_heads=5, lin_dim=7, lin_vdim=9,
+         decay=[0.9, 0.8, 0.7, 0.6, 1.0], ff=33),
 ]
 
 

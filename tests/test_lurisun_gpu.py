@@ -62,7 +62,7 @@ def test_pair_hash_embed(dt, W, buckets):
 
 @pytest.mark.parametrize("odt", DTS)
 @pytest.mark.parametrize("C,taps", [(64, 3), (36, 4), (1030, 2), (7, 1),
-                                    (130, 8)])
+                                    (130, 8), (50, 16)])
 def test_causal_conv_residual(odt, C, taps):
     torch.manual_seed(C + taps)
     T, B, Bc = 37, 3, 4
@@ -225,14 +225,14 @@ def test_mul_sigmoid_and_gated_activation(dt, N):
                                ref.swiglu(gu.cpu()).float(), **_tol(dt))
 
 
-def _executors(dtype, kw, mb=4, smax=256):
+def _executors(dtype, kw, mb=4, smax=256, width=96, vocab=200):
     from dnet_amd.models import ModelConfig
     from dnet_amd.models.config import lurisun_config
     from dnet_amd.parallel.ring import RingExecutor
     from lurisun_oracle import make_checkpoint
     # bfloat16: the two paths round differently and every layer of a random
     # stack multiplies that noise, so the bfloat16 stack is shallow
-    hf = lurisun_config(96, 200, "nla",
+    hf = lurisun_config(width, vocab, "nla",
                         layers=6 if dtype == "float32" else 3, **kw)
     sd = make_checkpoint(hf, seed=11)
     out = []
@@ -279,3 +279,30 @@ def test_model_gpu_equals_cpu(dtype, kw):
     assert rel < (2e-4 if dtype == "float32" else 0.1), rel
     worst = float((gpu - cpu).abs().max() / cpu.abs().max())
     assert worst < (1e-3 if dtype == "float32" else 0.3), worst
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_odd_sizes_gpu_matches_cpu(dtype):
+    """Sizes that are multiples of nothing (width, vocabulary, ranks, head
+    sizes, feed-forward width) and sixteen heads on one latent: every
+    kernel's unvectorized path and the linears' fallbacks, prompt and
+    decode."""
+    kw = dict(heads=3, kv_heads=1, dim=13, rot_dims=6, chunk=9,
+              latent_heads=16, latent_dim=7, latent_vdim=5, kv_rank=21,
+              q_rank=11, window=6, lin_heads=3, lin_dim=9, lin_vdim=11,
+              decay=[0.9, 1.0, 0.3], ff=37, taps=5, buckets=101)
+    prompts = [torch.arange(19) % 77, (torch.arange(3) * 7) % 77]
+    outs = []
+    for ex in _executors(dtype, kw, mb=2, smax=64, width=50, vocab=77):
+        rows = [r.float().cpu() for r in ex.prefill_slots(
+            [1, 0], prompts, want=[list(range(19)), [2]])]
+        for step in range(3):
+            ex.tokbuf[0].copy_(torch.tensor([5 + step, 9 + step]))
+            ex.slot_step_compute(park=torch.zeros(2, dtype=torch.bool,
+                                                  device=ex.device))
+            rows.append(ex.logits_buf[0].float().cpu().clone())
+            ex.kvs[0].pos.add_(1)
+        outs.append(torch.cat(rows))
+    cpu, gpu = outs
+    rel = float((gpu - cpu).pow(2).mean().sqrt() / cpu.pow(2).mean().sqrt())
+    assert rel < (2e-4 if dtype == "float32" else 0.2), rel
