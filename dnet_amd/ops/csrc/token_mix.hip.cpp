@@ -95,9 +95,10 @@ template <> __device__ __forceinline__ void ld4<short>(const short* p, float (&v
 template <typename T, bool V4>
 __global__ __launch_bounds__(256) void pair_hash_embed_kernel(
     const int64_t* __restrict__ tokens, const T* __restrict__ embed,
-    const T* __restrict__ table, const int* __restrict__ prev,
+    const T* __restrict__ table, const int* prev,
     float* __restrict__ out, const Rows g, const int W, const int vocab,
-    const int buckets, const int64_t mul_prev, const int64_t mul_cur) {
+    const int buckets, const int64_t mul_prev, const int64_t mul_cur,
+    int* prev_out) {
   const int64_t row = blockIdx.x;
   const int b = (int)(row / g.T), t = (int)(row % g.T);
   int p0, n, slot;
@@ -113,6 +114,12 @@ __global__ __launch_bounds__(256) void pair_hash_embed_kernel(
       pr = (last * mul_prev + tok * mul_cur) % buckets;
       if (pr < 0) pr += buckets;
     }
+  }
+  if (prev_out != nullptr) {
+    // one token per row (decode): this workgroup alone reads the slot's last
+    // token, so it also moves it on, once every thread has read it
+    __syncthreads();
+    if (on && threadIdx.x == 0) prev_out[slot] = (int)tokens[row];
   }
   const T* er = embed + tok * W;
   const T* tr = pr >= 0 ? table + pr * W : nullptr;
@@ -134,8 +141,9 @@ __global__ __launch_bounds__(256) void pair_hash_embed_kernel(
   }
 }
 
-// grid (B): after the rows are embedded, the slot's last token moves on.
-// A separate launch: every row of the embed kernel reads the old value.
+// grid (B), prompts only: after the rows are embedded, the slot's last token
+// moves on. A separate launch: every row of the embed kernel reads the old
+// value.
 __global__ void pair_hash_state_kernel(const int64_t* __restrict__ tokens,
                                        int* __restrict__ prev, const Rows g,
                                        const int B) {
@@ -152,11 +160,14 @@ __global__ void pair_hash_state_kernel(const int64_t* __restrict__ tokens,
 constexpr int kTile = 16;
 constexpr int kMaxTaps = 16;
 
-template <typename TO>
+// TAIL (a row's tokens fit one tile, decode steps above all): the thread that
+// walked the row also writes the slot's new tail, which is what its window
+// registers hold at the end; otherwise conv_tail_kernel does, in a launch of
+// its own, after every tile has read the old tail.
+template <typename TO, bool TAIL>
 __global__ __launch_bounds__(256) void conv_residual_kernel(
-    const float* __restrict__ x, const float* __restrict__ w,
-    const float* __restrict__ state, TO* __restrict__ y, const Rows g,
-    const int C, const int taps) {
+    const float* __restrict__ x, const float* __restrict__ w, float* state,
+    TO* __restrict__ y, const Rows g, const int C, const int taps) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= C) return;
   const int ntile = (g.T + kTile - 1) / kTile;
@@ -203,6 +214,15 @@ __global__ __launch_bounds__(256) void conv_residual_kernel(
       }
     }
     stx<TO>(y + row * C + c, acc);
+  }
+  if constexpr (TAIL) {
+    if (valid) {
+#pragma unroll
+      for (int j = 0; j < kMaxTaps - 1; ++j) {
+        if (j >= taps - 1) break;
+        state[((int64_t)slot * (taps - 1) + j) * C + c] = win[j];
+      }
+    }
   }
 }
 
@@ -453,13 +473,15 @@ void pair_hash_embed(torch::Tensor tokens, torch::Tensor embed,
                      tokens.data_ptr<int64_t>(), (const TT*)embed.data_ptr(),  \
                      (const TT*)table.data_ptr(), prev.data_ptr<int>(),        \
                      out.data_ptr<float>(), g, W, (int)embed.size(0),          \
-                     (int)buckets, mul_prev, mul_cur)
+                     (int)buckets, mul_prev, mul_cur,                          \
+                     T == 1 ? prev.data_ptr<int>() : nullptr)
   const bool v4 = W % 4 == 0;
   if (is_bf16(embed)) { if (v4) PE(short, true); else PE(short, false); }
   else if (is_f32(embed)) { if (v4) PE(float, true); else PE(float, false); }
   else DNET_CHECK(false, "pair_hash_embed: dtype");
 #undef PE
-  hipLaunchKernelGGL(pair_hash_state_kernel, dim3((unsigned)((B + 63) / 64)),
+  if (T > 1)
+    hipLaunchKernelGGL(pair_hash_state_kernel, dim3((unsigned)((B + 63) / 64)),
                      dim3(64), 0, st, tokens.data_ptr<int64_t>(),
                      prev.data_ptr<int>(), g, (int)B);
 }
@@ -486,18 +508,16 @@ void causal_conv_residual(torch::Tensor x, torch::Tensor w, torch::Tensor state,
   auto st = current_stream();
   const int ntile = (int)((T + kTile - 1) / kTile);
   const dim3 grid((unsigned)((C + 255) / 256), (unsigned)(B * ntile));
-  if (is_bf16(y))
-    hipLaunchKernelGGL((conv_residual_kernel<short>), grid, dim3(256), 0, st,
-                       x.data_ptr<float>(), w.data_ptr<float>(),
-                       state.data_ptr<float>(), (short*)y.data_ptr(), g, C,
-                       taps);
-  else if (is_f32(y))
-    hipLaunchKernelGGL((conv_residual_kernel<float>), grid, dim3(256), 0, st,
-                       x.data_ptr<float>(), w.data_ptr<float>(),
-                       state.data_ptr<float>(), (float*)y.data_ptr(), g, C,
-                       taps);
+  const bool fused = ntile == 1;        // the walking thread writes the tail
+#define CR(TT, FF)                                                            \
+  hipLaunchKernelGGL((conv_residual_kernel<TT, FF>), grid, dim3(256), 0, st,  \
+                     x.data_ptr<float>(), w.data_ptr<float>(),                \
+                     state.data_ptr<float>(), (TT*)y.data_ptr(), g, C, taps)
+  if (is_bf16(y)) { if (fused) CR(short, true); else CR(short, false); }
+  else if (is_f32(y)) { if (fused) CR(float, true); else CR(float, false); }
   else DNET_CHECK(false, "causal_conv_residual: output dtype");
-  if (taps > 1)
+#undef CR
+  if (taps > 1 && !fused)
     hipLaunchKernelGGL(conv_tail_kernel,
                        dim3((unsigned)((C + 255) / 256), (unsigned)B),
                        dim3(256), 0, st, x.data_ptr<float>(),
